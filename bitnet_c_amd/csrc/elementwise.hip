@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void rmsnorm_ssq_kernel(const float* __restric
 // out[r, :] = x[rows[r], :] in type T: the wanted rows of the stream for an output matrix that no norm precedes
 template <typename T>
 __global__ void gather_rows_kernel(T* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows, int dim) {
-    const float* xr = x + (size_t)rows[blockIdx.x] * dim;
+    const float* xr = x + (size_t)(rows ? rows[blockIdx.x] : (int)blockIdx.x) * dim;       // rows null: every row in turn
     T* o = out + (size_t)blockIdx.x * dim;
     for (int i = threadIdx.x; i < dim; i += blockDim.x) o[i] = from_f32<T>(xr[i]);
 }
@@ -337,7 +337,7 @@ extern "C" int bn_embed_gather(int dtype, void* x, const void* table, const int*
 
 // out [n_rows, dim] (dtype) = the rows `rows` of x [., dim] (float32)
 extern "C" int bn_gather_rows(int dtype, void* out, const float* x, const int* rows, int n_rows, int dim, hipStream_t s) {
-    if (n_rows <= 0 || dim <= 0 || !out || !x || !rows) return BN_ERR_ARG;
+    if (n_rows <= 0 || dim <= 0 || !out || !x) return BN_ERR_ARG;
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(gather_rows_kernel<float>, dim3(n_rows), dim3(256), 0, s, (float*)out, x, rows, dim);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(gather_rows_kernel<bf16>, dim3(n_rows), dim3(256), 0, s, (bf16*)out, x, rows, dim);
     else return BN_ERR_DTYPE;
@@ -656,16 +656,20 @@ __global__ void add_normed_rmsnorm_kernel(float* __restrict__ x, const TD* __res
         sx = fmaf(v, v, sx);
     }
     if (!out) return;
+    T* o = out + (size_t)r * dim;
+    if (!w) {                                            // every thread reads back what it wrote itself
+        for (int i = threadIdx.x; i < dim; i += blockDim.x) o[i] = from_f32<T>(row[i]);
+        return;
+    }
     sx = block_sum(sx, scratch);
     const float f = 1.0f / sqrtf(sx / (float)dim + eps);
-    T* o = out + (size_t)r * dim;
     for (int i = threadIdx.x; i < dim; i += blockDim.x) o[i] = from_f32<T>(row[i] * f * w[i]);
 }
 
 // dtype: the type of out (and of delta when parts_f32 is 0); parts_f32: delta is n_parts float32 slabs [n_parts][n_rows][dim]
 extern "C" int bn_add_normed_rmsnorm(int dtype, void* x, const void* delta, int n_parts, int parts_f32, const float* wb,
                                      float eps_b, const float* w, void* out, int n_rows, int dim, float eps, hipStream_t s) {
-    if (n_rows <= 0 || dim <= 0 || dim > 16384 || n_parts < 1 || !x || !delta || !wb || ((w == nullptr) != (out == nullptr)))
+    if (n_rows <= 0 || dim <= 0 || dim > 16384 || n_parts < 1 || !x || !delta || !wb || (w && !out))
         return BN_ERR_ARG;
     if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
     const int threads = dim >= 2048 ? 512 : 256;

@@ -1,7 +1,12 @@
-// A mixture-of-experts feed-forward whose experts have no gate: expert e is  W_down[e] act(W_up[e] x).
+// A mixture-of-experts feed-forward.  Expert e is  W_down[e] act(W_up[e] x)  (no gate), or, in the gated form,
+// W_down[e] glu(W_gate[e] x, W_up[e] x)  with the clamped unit  glu(g, u) = g' sigmoid(slope g') (u' + shift),
+// g' = min(g, limit), u' = clamp(u, -limit, limit)  (gate and up rows stacked, [E, 2 F, D]).
 //
 //   bn_moe_route     router logits z = W_r h in float32 (one workgroup a token), scores sigmoid(z) or softmax(z), the top_k
-//                    largest (ties: the lower index), optionally divided by their sum -> expert ids and weights [T, top_k]
+//                    largest (ties: the lower index; with a choice bias the largest score + bias, the weights staying the
+//                    plain scores), optionally divided by their sum (+ floor), times a constant -> expert ids and weights
+//                    [T, top_k]; optionally also sigmoid(w_g . h) per token, the gate of a shared expert
+//   bn_gated_unit    rows of stacked (gate | up) products -> the clamped unit, optionally times a factor per row
 //   bn_moe_experts   for every (token, choice) pair: y = W_down[e] act(W_up[e] (w h)) when the weight multiplies the
 //                    expert's input, w * W_down[e] act(W_up[e] h) when it multiplies the output; a pair reads its expert's
 //                    two matrices once, their rows spread over workgroups.  The products accumulate in float32; the scaled
@@ -24,6 +29,10 @@ struct RouteArgs {
     int* ids;                 // [T, K]
     float* wts;               // [T, K]
     int ld, D, E, K, scoring, renorm;
+    const float* bias;        // [E] added to the scores for the choice alone; null: the choice goes by the scores
+    const float* gate_w;      // [D]: gate_out[t] = sigmoid(gate_w . h); null: none
+    float* gate_out;          // [T]
+    float floor, scale;       // weights = score / (sum of the chosen + floor) (when renorm) * scale
 };
 
 #define MOE_ROUTE_THREADS 256
@@ -38,8 +47,9 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
     const T* h = reinterpret_cast<const T*>(a.h) + (size_t)t * a.ld;
     for (int d = threadIdx.x; d < a.D; d += MOE_ROUTE_THREADS) hs[d] = to_f32(h[d]);
     __syncthreads();
-    for (int e = wave; e < a.E; e += MOE_ROUTE_THREADS / BN_WAVE) {
-        const float* w = a.wr + (size_t)e * a.D;
+    // the shared expert's gate is one more row: it takes its turn among the waves after the experts
+    for (int e = wave; e < a.E + (a.gate_w ? 1 : 0); e += MOE_ROUTE_THREADS / BN_WAVE) {
+        const float* w = e < a.E ? a.wr + (size_t)e * a.D : a.gate_w;
         float s = 0.f;
         if (a.D % 4 == 0) {
 #pragma unroll 4
@@ -51,7 +61,10 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
             for (int d = lane; d < a.D; d += BN_WAVE) s = fmaf(hs[d], w[d], s);
         }
         s = wave_sum(s);
-        if (lane == 0) zs[e] = s;
+        if (lane == 0) {
+            if (e < a.E) zs[e] = s;
+            else a.gate_out[t] = 1.0f / (1.0f + expf(-s));
+        }
     }
     __syncthreads();
     if (wave != 0) return;
@@ -68,6 +81,20 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
         for (int j = 0; j < MOE_PER_LANE; ++j) sum += z[j] == -INFINITY ? 0.f : expf(z[j] - zmax);
         denom = wave_sum(sum);
     }
+    // with a choice bias the experts are ranked by score + bias: the scores of all experts are formed first and z holds
+    // the ranking value from here on
+    float sc[MOE_PER_LANE];
+    if (a.bias) {
+#pragma unroll
+        for (int j = 0; j < MOE_PER_LANE; ++j) {
+            const int e = lane + BN_WAVE * j;
+            sc[j] = 0.f;
+            if (e < a.E) {
+                sc[j] = a.scoring == MOE_SCORE_SOFTMAX ? expf(z[j] - zmax) / denom : 1.0f / (1.0f + expf(-z[j]));
+                z[j] = sc[j] + a.bias[e];
+            }
+        }
+    }
     float total = 0.f, mine_w = 0.f;
     int mine_id = 0;
     for (int k = 0; k < a.K; ++k) {
@@ -83,10 +110,12 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
             if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
         }
         if (at >= a.E) at = k;                           // a row of NaNs (a padding row's garbage): still an expert that exists
+        float own = 0.f;                                 // the chosen expert's plain score, held by the lane that owns it
 #pragma unroll
         for (int j = 0; j < MOE_PER_LANE; ++j)
-            if (at == lane + BN_WAVE * j) z[j] = -INFINITY;
-        const float score = a.scoring == MOE_SCORE_SOFTMAX ? expf(best - zmax) / denom : 1.0f / (1.0f + expf(-best));
+            if (at == lane + BN_WAVE * j) { z[j] = -INFINITY; if (a.bias) own = sc[j]; }
+        const float score = a.bias ? wave_sum(own)
+                          : a.scoring == MOE_SCORE_SOFTMAX ? expf(best - zmax) / denom : 1.0f / (1.0f + expf(-best));
         total += score;
         if (lane == k % BN_WAVE && k < BN_WAVE) { mine_w = score; mine_id = at; }
         if (k >= BN_WAVE && lane == 0) {                  // more choices than lanes: stored as they come
@@ -94,23 +123,26 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
             a.wts[(size_t)t * a.K + k] = score;
         }
     }
-    const float norm = a.renorm ? 1.0f / total : 1.0f;
+    const float norm = (a.renorm ? 1.0f / (total + a.floor) : 1.0f) * a.scale;
     if (lane < a.K) {
         a.ids[(size_t)t * a.K + lane] = mine_id;
         a.wts[(size_t)t * a.K + lane] = mine_w * norm;
     }
-    if (a.renorm && a.K > BN_WAVE && lane == 0)
+    if ((a.renorm || a.scale != 1.0f) && a.K > BN_WAVE && lane == 0)
         for (int k = BN_WAVE; k < a.K; ++k) a.wts[(size_t)t * a.K + k] *= norm;
 }
 
 extern "C" int bn_moe_route(int dtype, const void* h, int ld, const float* wr, int* ids, float* wts, int n_tokens, int D, int E,
-                            int K, int scoring, int renorm, hipStream_t s) {
+                            int K, int scoring, int renorm, const float* bias, float floor, float scale, const float* gate_w,
+                            float* gate_out, hipStream_t s) {
+    if ((gate_w == nullptr) != (gate_out == nullptr) || ((uintptr_t)gate_w & 15) || !(floor >= 0.f)) return BN_ERR_ARG;
     if (n_tokens <= 0 || D <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || K <= 0 || K > E || ld < D || !h || !wr || !ids || !wts)
         return BN_ERR_ARG;
     if (scoring != MOE_SCORE_SIGMOID && scoring != MOE_SCORE_SOFTMAX) return BN_ERR_ARG;
     if ((size_t)(D + 4 + E) * sizeof(float) > 64 * 1024 || ((uintptr_t)wr & 15)) return BN_ERR_ARG;
     RouteArgs a;
     a.h = h; a.wr = wr; a.ids = ids; a.wts = wts; a.ld = ld; a.D = D; a.E = E; a.K = K; a.scoring = scoring; a.renorm = renorm ? 1 : 0;
+    a.bias = bias; a.gate_w = gate_w; a.gate_out = gate_out; a.floor = floor; a.scale = scale;
     const size_t shm = (size_t)(((D + 3) & ~3) + E) * sizeof(float);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(MOE_ROUTE_THREADS), shm, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(MOE_ROUTE_THREADS), shm, s, a);
@@ -135,7 +167,16 @@ struct PairArgs {
     float* hidden;            // [T K, F] float32 holding values of the activations' type
     float* y;                 // [K, T, D]
     int ld, T, D, F, K, act, weight_on_input;      // T: the rows of a slab of y
+    int gated;                // w_up is [E, 2 F, D]: F gate rows, then F up rows; hidden = the clamped unit of the two
+    float limit, slope, shift;
 };
+
+// the clamped gated unit: g' sigmoid(slope g') (u' + shift), g' = min(g, limit), u' = clamp(u, -limit, limit)
+__device__ __forceinline__ float moe_clamped_unit(float g, float u, float limit, float slope, float shift) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-slope * g)) * (u + shift);
+}
 
 // sum over n of x[i] w[i]: x in shared memory, w a row in global memory; every lane gets the sum
 template <typename T>
@@ -174,8 +215,27 @@ __global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_up_kernel(PairArgs 
     const T* h = reinterpret_cast<const T*>(a.h) + (size_t)t * a.ld;
     for (int d = threadIdx.x; d < a.D; d += MOE_PAIR_THREADS) xs[d] = to_f32(from_f32<T>(to_f32(h[d]) * in_scale));
     __syncthreads();
-    const T* wu = reinterpret_cast<const T*>(a.w_up) + (size_t)e * a.F * a.D;
+    const T* wu = reinterpret_cast<const T*>(a.w_up) + (size_t)e * (a.gated ? 2 : 1) * a.F * a.D;
     const int f0 = blockIdx.x * MOE_PAIR_ROWS;
+    if (a.gated) {
+        // a gate row and its up row one after the other, both rows' loads in flight; the products are rounded to the
+        // activations' type, as the rows of a stacked product of that type are, before they meet in the unit
+        float g[MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE)], u[MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE)];
+#pragma unroll
+        for (int k = 0; k < MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE); ++k) {
+            const int f = f0 + wave + k * (MOE_PAIR_THREADS / BN_WAVE);
+            g[k] = f < a.F ? moe_row_dot<T>(wu + (size_t)f * a.D, xs, a.D, lane) : 0.f;
+            u[k] = f < a.F ? moe_row_dot<T>(wu + (size_t)(a.F + f) * a.D, xs, a.D, lane) : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE); ++k) {
+            const int f = f0 + wave + k * (MOE_PAIR_THREADS / BN_WAVE);
+            if (f < a.F && lane == 0)
+                a.hidden[(size_t)pair * a.F + f] = to_f32(from_f32<T>(moe_clamped_unit(
+                    to_f32(from_f32<T>(g[k])), to_f32(from_f32<T>(u[k])), a.limit, a.slope, a.shift)));
+        }
+        return;
+    }
     // a wave's two rows (MOE_PAIR_ROWS / 4) one after the other without a dependence between them: both rows' loads are
     // in flight before the first sum is needed
     float sums[MOE_PAIR_ROWS / (MOE_PAIR_THREADS / BN_WAVE)];
@@ -221,13 +281,15 @@ __global__ __launch_bounds__(MOE_PAIR_THREADS) void moe_pair_down_kernel(PairArg
 // step's tokens, y then points at the run's first row of slab 0)
 extern "C" int bn_moe_experts(int dtype, const void* h, int ld, const void* w_up, const void* w_down, const int* ids,
                               const float* wts, float* y, float* hidden, int n_tokens, int y_rows, int D, int F, int K, int act,
-                              int weight_on_input, hipStream_t s) {
-    if (n_tokens <= 0 || y_rows < n_tokens || D <= 0 || F <= 0 || K <= 0 || ld < D || act < 0 || act >= BN_UNARY_KINDS) return BN_ERR_ARG;
+                              int weight_on_input, int gated, float limit, float slope, float shift, hipStream_t s) {
+    if (n_tokens <= 0 || y_rows < n_tokens || D <= 0 || F <= 0 || K <= 0 || ld < D) return BN_ERR_ARG;
+    if (gated ? !(limit > 0.f) : (act < 0 || act >= BN_UNARY_KINDS)) return BN_ERR_ARG;
     if (!h || !w_up || !w_down || !ids || !wts || !y || !hidden) return BN_ERR_ARG;
     if ((size_t)D * sizeof(float) > 64 * 1024 || (size_t)F * sizeof(float) > 64 * 1024 || (size_t)n_tokens * K > 65535) return BN_ERR_ARG;
     PairArgs a;
     a.h = h; a.w_up = w_up; a.w_down = w_down; a.ids = ids; a.wts = wts; a.y = y; a.hidden = hidden;
     a.ld = ld; a.T = y_rows; a.D = D; a.F = F; a.K = K; a.act = act; a.weight_on_input = weight_on_input ? 1 : 0;
+    a.gated = gated ? 1 : 0; a.limit = limit; a.slope = slope; a.shift = shift;
     const dim3 block(MOE_PAIR_THREADS);
     const dim3 up((F + MOE_PAIR_ROWS - 1) / MOE_PAIR_ROWS, n_tokens * K), down((D + MOE_PAIR_ROWS - 1) / MOE_PAIR_ROWS, n_tokens * K);
     if (dtype == BN_DT_F32) {
@@ -325,5 +387,33 @@ extern "C" int bn_moe_group(const void* h, int ld, const int* ids, const float* 
     hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(MOE_PLAN_THREADS), 0, s, ids, n_pairs, E, tile_rows, order, tiles, n_tiles);
     hipLaunchKernelGGL(moe_gather_kernel, dim3(n_pairs), dim3(256), 0, s, (const bf16*)h, ld, order, wts, (bf16*)xg, row_map,
                        row_scale, n_tokens, D, K, scale_input ? 1 : 0);
+    return bn_launch_status();
+}
+
+// ---- the clamped gated unit over rows of stacked products ------------------------------------------------------------
+// out[r, f] = unit(gu[r, f], gu[r, F + f]) (times row_scale[r]), rounded once to the activations' type: what follows a
+// product with stacked gate and up rows, for the grouped experts and for a shared expert (whose factor is its gate)
+template <typename T>
+__global__ void gated_unit_kernel(T* __restrict__ out, const T* __restrict__ gu, int ld, const float* __restrict__ row_scale,
+                                  int n_rows, int F, float limit, float slope, float shift) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (size_t)n_rows * F) return;
+    const int r = (int)(i / F), f = (int)(i - (size_t)r * F);
+    const T* row = gu + (size_t)r * ld;
+    float v = moe_clamped_unit(to_f32(row[f]), to_f32(row[F + f]), limit, slope, shift);
+    if (row_scale) v *= row_scale[r];
+    out[i] = from_f32<T>(v);
+}
+
+extern "C" int bn_gated_unit(int dtype, void* out, const void* gu, int ld, const float* row_scale, int n_rows, int F, float limit,
+                             float slope, float shift, hipStream_t s) {
+    if (n_rows <= 0 || F <= 0 || ld < 2 * F || !out || !gu || !(limit > 0.f)) return BN_ERR_ARG;
+    const size_t n = (size_t)n_rows * F;
+    const dim3 grid((unsigned)((n + 255) / 256)), block(256);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(gated_unit_kernel<float>, grid, block, 0, s, (float*)out, (const float*)gu, ld, row_scale, n_rows, F, limit, slope, shift);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(gated_unit_kernel<bf16>, grid, block, 0, s, (bf16*)out, (const bf16*)gu, ld, row_scale, n_rows, F, limit, slope, shift);
+    else return BN_ERR_DTYPE;
     return bn_launch_status();
 }

@@ -10,6 +10,9 @@
 //   k_g <- rot_p(k_g / rms * wk)                       -> page of position p
 //   v_g                                                 -> page of position p
 //
+// v_from_k: the values are the key projections themselves, as projected (before the key's norm and rotation): qkv then
+// holds no value heads, and kv head g's value is read from its key's columns, which this kernel leaves as they arrived.
+//
 // Pages hold a row per position for the keys, [page, kv head, BN_PAGE, hs]; the values lie the same way ("rows" layout,
 // [page, kv head, BN_PAGE, vd]) or transposed ([page, kv head, vd, BN_PAGE]), as the caller says.
 #include "common.h"
@@ -34,6 +37,7 @@ struct QkNormArgs {
     int rope_dims, rope_interleaved;
     float eps, temp_coef;
     int temp_every;           // <= 0: no temperature
+    int v_from_k;             // the values are the keys as projected (vd == hs; qkv has no value columns)
 };
 
 // sine and cosine of an angle of any size: the angle less the nearest multiple of 2 pi (2 pi as the sum of two floats, the
@@ -122,7 +126,7 @@ __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNo
         } else {
             if (!a.v_pages) continue;
             const int kvh = head - a.H - a.Hkv;
-            const T* v = row + (size_t)(a.H + a.Hkv) * a.hs + (size_t)kvh * a.vd;
+            const T* v = a.v_from_k ? row + (size_t)(a.H + kvh) * a.hs : row + (size_t)(a.H + a.Hkv) * a.hs + (size_t)kvh * a.vd;
             const int page = a.block_table[(size_t)a.seq_index[t] * a.bt_stride + pos / BN_PAGE];
             if (a.v_transposed) {
                 T* dst = reinterpret_cast<T*>(a.v_pages) + ((size_t)page * a.Hkv + kvh) * a.vd * BN_PAGE + pos % BN_PAGE;
@@ -139,10 +143,10 @@ extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positio
                                 const int* block_table, int bt_stride, void* k_pages, void* v_pages, const float* wq,
                                 const float* wk, int n_tokens, int H, int Hkv, int hs, int vd, float eps, float temp_coef,
                                 int temp_every, int v_transposed, int norm_all, const float* inv_freq, int rope_dims,
-                                int rope_interleaved, hipStream_t s) {
+                                int rope_interleaved, int v_from_k, hipStream_t s) {
     if (n_tokens <= 0 || H <= 0 || Hkv <= 0 || hs <= 0 || hs > BN_MAX_HEAD_DIM || vd <= 0 || !qkv || !positions) return BN_ERR_ARG;
     if ((k_pages == nullptr) != (v_pages == nullptr) || (k_pages && (!seq_index || !block_table))) return BN_ERR_ARG;
-    if ((wq == nullptr) != (wk == nullptr) || ld < H * hs + Hkv * (hs + vd)) return BN_ERR_ARG;
+    if ((wq == nullptr) != (wk == nullptr) || ld < H * hs + Hkv * (v_from_k ? hs : hs + vd) || (v_from_k && vd != hs)) return BN_ERR_ARG;
     if (inv_freq && (rope_dims <= 0 || rope_dims % 2 || rope_dims > hs)) return BN_ERR_ARG;
     QkNormArgs a;
     a.qkv = qkv; a.positions = positions; a.seq_index = seq_index; a.block_table = block_table;
@@ -150,6 +154,7 @@ extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positio
     a.ld = ld; a.bt_stride = bt_stride; a.H = H; a.Hkv = Hkv; a.hs = hs; a.vd = vd;
     a.eps = eps; a.temp_coef = temp_coef; a.temp_every = temp_every; a.v_transposed = v_transposed ? 1 : 0;
     a.norm_all = norm_all ? 1 : 0; a.rope_dims = inv_freq ? rope_dims : 0; a.rope_interleaved = rope_interleaved ? 1 : 0;
+    a.v_from_k = v_from_k ? 1 : 0;
     const dim3 grid(n_tokens, (H + 2 * Hkv + QKN_WAVES - 1) / QKN_WAVES), block(QKN_WAVES * BN_WAVE);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, 0, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, block, 0, s, a);

@@ -55,7 +55,7 @@ _SIGNATURES = {
     "qk_norm": {
         "bn_qk_norm_store": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                              c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int, c_int, c_int, c_void_p, c_int,
-                             c_int, c_void_p],
+                             c_int, c_int, c_void_p],
     },
     "latent": {
         "bn_latent_store": [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
@@ -66,9 +66,10 @@ _SIGNATURES = {
     },
     "moe": {
         "bn_moe_route": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_void_p],
+                         c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p],
         "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                           c_int, c_int, c_int, c_int, c_void_p],
+                           c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p],
+        "bn_gated_unit": [c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_float, c_float, c_void_p],
         "bn_moe_grouped_tiles": [c_int, c_int, c_int],
         "bn_moe_group": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                          c_int, c_void_p],
@@ -80,6 +81,12 @@ _SIGNATURES = {
         "bn_attn_general_decode": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
                                    c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
                                    c_void_p, c_void_p, c_void_p],
+    },
+    "lightning": {
+        "bn_lightning_supports": [c_int, c_int],
+        "bn_lightning_scan": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
+                              c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bn_row_norm_gate": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     },
     "state_mixers": {
         "bn_token_shift": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
@@ -267,6 +274,20 @@ def gather_rows(x: torch.Tensor, rows: torch.Tensor, out_dtype) -> torch.Tensor:
     if rows.numel():
         _check(_fn("elementwise", "bn_gather_rows")(_code(out_dtype), out.data_ptr(), x.data_ptr(), rows.data_ptr(), rows.numel(),
                                                     x.shape[1], _stream()), "gather_rows")
+    return out
+
+
+def stream_rows(x: torch.Tensor, out_dtype) -> torch.Tensor:
+    """Every row of the float32 stream x [T, D] in out_dtype (a copy): what a part reads when no norm stands in front
+    of it."""
+    require_gpu()
+    _dev(x, "x", torch.float32, 2)
+    if not x.is_contiguous():
+        raise KernelError("stream_rows: x must be contiguous")
+    out = torch.empty(tuple(x.shape), dtype=out_dtype, device=x.device)
+    if x.shape[0]:
+        _check(_fn("elementwise", "bn_gather_rows")(_code(out_dtype), out.data_ptr(), x.data_ptr(), None, x.shape[0], x.shape[1],
+                                                    _stream()), "stream_rows")
     return out
 
 
@@ -1343,7 +1364,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
 def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, hs: int, *, v_dim: int = 0,
                   q_weight=None, k_weight=None, eps: float = 0.0, temp_coef: float = 0.0, temp_every: int = 0,
                   seq_index=None, block_table=None, k_pages=None, v_pages=None, v_transposed: bool = False,
-                  norm_projection: bool = False, inv_freq=None, rope_dims: int = 0, rope_interleaved: bool = False) -> None:
+                  norm_projection: bool = False, inv_freq=None, rope_dims: int = 0, rope_interleaved: bool = False,
+                  v_from_k: bool = False) -> None:
     """In place on qkv [T, H hs + Hkv (hs + v_dim)]: every query and key head under an RMSNorm of its own (weights
     [hs] float32, shared by the heads; both or neither), or, with norm_projection, one RMSNorm over the whole query
     projection and one over the whole key projection (weights [H hs] and [Hkv hs]); then the first rope_dims dimensions
@@ -1351,13 +1373,17 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
     rope_interleaved, (i, i + rope_dims / 2) otherwise; inv_freq None: no rotation); the queries times
     1 + temp_coef ln(floor((p + 1) / temp_every) + 1) at position p (temp_every 0: no temperature); the keys and the
     values go into the pages when pages are given (keys a row per position; values the same way, or transposed inside a
-    page when v_transposed).  Rows with position < 0 are left alone."""
+    page when v_transposed).  Rows with position < 0 are left alone.  v_from_k: the values are the key projections as
+    they arrived (before norm and rotation); qkv is [T, (H + Hkv) hs] then and v_dim equals hs."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(positions, "positions", torch.int32, 1)
     vd = int(v_dim) or hs
     T = qkv.shape[0]
-    if positions.numel() != T or qkv.shape[1] < H * hs + Hkv * (hs + vd) or (q_weight is None) != (k_weight is None):
+    if v_from_k and vd != hs:
+        raise KernelError(f"qk_norm_store: values that are the keys are as wide as the keys, got {vd} and {hs}")
+    if (positions.numel() != T or qkv.shape[1] < H * hs + Hkv * (hs if v_from_k else hs + vd)
+            or (q_weight is None) != (k_weight is None)):
         raise KernelError(f"qk_norm_store: qkv {tuple(qkv.shape)} does not fit H={H} Hkv={Hkv} hs={hs} v_dim={vd}")
     for w, nm, heads in ((q_weight, "q_weight", H), (k_weight, "k_weight", Hkv)):
         if w is not None:
@@ -1386,8 +1412,8 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
         v_pages.data_ptr() if k_pages is not None else None, q_weight.data_ptr() if q_weight is not None else None,
         k_weight.data_ptr() if k_weight is not None else None, T, H, Hkv, hs, vd, float(eps), float(temp_coef),
         int(temp_every), int(bool(v_transposed)), int(bool(norm_projection)),
-        inv_freq.data_ptr() if inv_freq is not None else None, int(rope_dims), int(bool(rope_interleaved)), _stream()),
-        "qk_norm_store")
+        inv_freq.data_ptr() if inv_freq is not None else None, int(rope_dims), int(bool(rope_interleaved)),
+        int(bool(v_from_k)), _stream()), "qk_norm_store")
 
 
 GENERAL_PROMPT_TILE = 16       # query tokens of a tile of attention_general_prompt
@@ -1748,12 +1774,71 @@ def mingru_scan(zxg: torch.Tensor, bias_z, bias_x, state: torch.Tensor, slot_ids
 # a part's output with a norm of its own; latent attention; mixture of experts
 # --------------------------------------------------------------------------------------
 
+LIGHTNING_MAX_DIM = _build.header_constant("LA_MAX_DIM", "lightning.hip")
+
+
+def lightning_supported(dk: int, dv: int) -> bool:
+    return 1 <= dk <= LIGHTNING_MAX_DIM and dv >= 1
+
+
+def lightning_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, decay: torch.Tensor, state: torch.Tensor, slot_ids,
+                   H: int, dk: int, dv: int, *, tiles=None, seq_lens=None) -> torch.Tensor:
+    """Linear attention with a fixed decay per head over every sequence of a step; float32 [T, H dv].  x [T, >= ...] in
+    the activations' type holds the projections side by side: queries at column q_col and keys at k_col (H dk wide),
+    values at v_col (H dv wide); each passes silu in float32.  decay [H] float32.  state [slots, >= H dk dv] float32, the
+    heads' matrices [H][dk][dv], updated in place; a sequence at position 0 starts from zeros.  Per head, in float32:
+        S <- decay S + k_t v_t^T;  o_t = S^T q_t."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(decay, "decay", torch.float32, 1)
+    T = x.shape[0]
+    if not lightning_supported(dk, dv):
+        raise KernelError(f"lightning_scan: key width up to {LIGHTNING_MAX_DIM}, got {dk} x {dv}")
+    ld = _rows(x, "x")
+    if (decay.numel() != H or not decay.is_contiguous() or min(q_col, k_col, v_col) < 0
+            or max(q_col + H * dk, k_col + H * dk, v_col + H * dv) > x.shape[1]):
+        raise KernelError(f"lightning_scan: x {tuple(x.shape)} does not hold H={H} heads of {dk} / {dv} at columns "
+                          f"{q_col}, {k_col}, {v_col}, or decay is not [H]")
+    stride = _state_rows(state, H * dk * dv, "lightning_scan")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    tl, n_seqs, sl = _seq_args(tiles, seq_lens, "lightning_scan")
+    if tiles is None and n_seqs != T:
+        raise KernelError("lightning_scan: a decode step has one length per row")
+    o = torch.empty((T, H * dv), dtype=torch.float32, device=x.device)
+    if T and n_seqs:
+        _check(_fn("lightning", "bn_lightning_scan")(_code(x.dtype), x.data_ptr(), ld, int(q_col), int(k_col), int(v_col),
+                                                     decay.data_ptr(), o.data_ptr(), state.data_ptr(), stride, tl, n_seqs, sl,
+                                                     slot_ids.data_ptr(), H, dk, dv, _stream()), "lightning_scan")
+    return o
+
+
+def row_norm_gate(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, activation: str = "sigmoid") -> torch.Tensor:
+    """o [T, W] float32 divided by its rows' root mean square (eps inside the root), times weight [W] (float32), times
+    act(gate) (gate [T, W] in the activations' type, which is the result's; act one of UNARY_ACTIVATIONS)."""
+    require_gpu()
+    _dev(o, "o", torch.float32, 2)
+    _dev(gate, "gate", dims=2)
+    _dev(weight, "weight", torch.float32, 1)
+    T, W = o.shape
+    if not o.is_contiguous() or tuple(gate.shape) != (T, W) or weight.numel() != W or not weight.is_contiguous():
+        raise KernelError("row_norm_gate: o and gate [T, W], weight [W]")
+    if activation not in UNARY_ACTIVATIONS:
+        raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
+    y = torch.empty((T, W), dtype=gate.dtype, device=o.device)
+    if T:
+        _check(_fn("lightning", "bn_row_norm_gate")(_code(gate.dtype), y.data_ptr(), o.data_ptr(), gate.data_ptr(),
+                                                    _rows(gate, "gate"), weight.data_ptr(), T, W, float(eps),
+                                                    UNARY_ACTIVATIONS[activation], _stream()), "row_norm_gate")
+    return y
+
+
 def add_normed_rmsnorm(x: torch.Tensor, delta, out_weight: torch.Tensor, out_eps: float, weight: Optional[torch.Tensor] = None,
-                       eps: float = 0.0, out_dtype=None):
+                       eps: float = 0.0, out_dtype=None, rows_out: bool = False):
     """x (float32, [T, D]) += out_weight * delta / sqrt(mean(delta^2) + out_eps), row by row in float32; delta [T, D]
     in x's or the activations' type, or PartialSums (its slabs are added first).  With `weight`, also returns the rows of
     the new x under an RMSNorm (weight, eps) in out_dtype: a block's output norm, the residual sum and the next part's
-    norm in one kernel."""
+    norm in one kernel.  rows_out (without weight): returns the rows of the new x themselves in out_dtype, for a next part
+    that reads the stream as it is."""
     require_gpu()
     _dev(x, "x", torch.float32, 2)
     _dev(out_weight, "out_weight", torch.float32, 1)
@@ -1768,10 +1853,13 @@ def add_normed_rmsnorm(x: torch.Tensor, delta, out_weight: torch.Tensor, out_eps
     if parts is None and d.dtype not in _DT:
         raise KernelError(f"add_normed_rmsnorm: unsupported delta type {d.dtype}")
     out = None
+    if weight is not None and rows_out:
+        raise KernelError("add_normed_rmsnorm: either the rows under a norm (weight) or the rows themselves (rows_out)")
     if weight is not None:
         _dev(weight, "weight", torch.float32, 1)
         if weight.numel() != D or not weight.is_contiguous():
             raise KernelError(f"add_normed_rmsnorm: weight must hold {D} values")
+    if weight is not None or rows_out:
         out = torch.empty((T, D), dtype=out_dtype or (torch.float32 if parts is not None else d.dtype), device=x.device)
     # the kernel's type names the type of out and of a delta that is no float32 slab
     code = _code(out.dtype) if out is not None else (_code(torch.float32) if parts is not None else _code(d.dtype))
@@ -1856,10 +1944,14 @@ MOE_SCORINGS = {"sigmoid": _build.header_constant("MOE_SCORE_SIGMOID", "moe.hip"
                 "softmax": _build.header_constant("MOE_SCORE_SOFTMAX", "moe.hip")}
 
 
-def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = "sigmoid", renormalize: bool = False):
+def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = "sigmoid", renormalize: bool = False, *,
+              choice_bias: Optional[torch.Tensor] = None, weight_floor: float = 0.0, weight_scale: float = 1.0,
+              gate: Optional[torch.Tensor] = None):
     """(ids [T, top_k] int32, weights [T, top_k] float32): router logits z = router . h in float32 (router [E, D]
     float32, h in the activations' type), scores sigmoid(z) or softmax(z) over the experts, the top_k largest in
-    descending order (ties: the lower index); renormalize divides the chosen scores by their sum."""
+    descending order (ties: the lower index); renormalize divides the chosen scores by their sum (+ weight_floor);
+    weight_scale multiplies the weights.  choice_bias [E] float32: the experts are chosen by score + bias, the weights
+    stay the plain scores.  gate [D] float32: a third result [T] float32, sigmoid(gate . h), a shared expert's gate."""
     require_gpu()
     _dev(h, "h", dims=2)
     _dev(router, "router", torch.float32, 2)
@@ -1870,38 +1962,90 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = 
     if router.shape[1] != D or not router.is_contiguous() or not 1 <= top_k <= E or E > MOE_MAX_EXPERTS or D > 16384:
         raise KernelError(f"moe_route: h {tuple(h.shape)}, router {tuple(router.shape)}, top_k {top_k} do not fit "
                           f"(at most {MOE_MAX_EXPERTS} experts, 16,384 columns)")
+    for t, nm, n in ((choice_bias, "choice_bias", E), (gate, "gate", D)):
+        if t is not None:
+            _dev(t, nm, torch.float32, 1)
+            if t.numel() != n or not t.is_contiguous():
+                raise KernelError(f"moe_route: {nm} must hold {n} float32 values")
+    if not weight_floor >= 0.0:
+        raise KernelError(f"moe_route: weight_floor {weight_floor} must not be negative")
     ids = torch.empty((T, top_k), dtype=torch.int32, device=h.device)
     wts = torch.empty((T, top_k), dtype=torch.float32, device=h.device)
+    gate_out = torch.empty((T,), dtype=torch.float32, device=h.device) if gate is not None else None
     if T:
         _check(_fn("moe", "bn_moe_route")(_code(h.dtype), h.data_ptr(), _rows(h, "h"), router.data_ptr(), ids.data_ptr(),
                                           wts.data_ptr(), T, D, E, int(top_k), MOE_SCORINGS[scoring], int(bool(renormalize)),
-                                          _stream()), "moe_route")
-    return ids, wts
+                                          choice_bias.data_ptr() if choice_bias is not None else None, float(weight_floor),
+                                          float(weight_scale), gate.data_ptr() if gate is not None else None,
+                                          gate_out.data_ptr() if gate is not None else None, _stream()), "moe_route")
+    return (ids, wts) if gate is None else (ids, wts, gate_out)
+
+
+@dataclass(frozen=True)
+class ClampedUnit:
+    """The gated unit glu(g, u) = g' sigmoid(slope g') (u' + shift) with g' = min(g, limit), u' = clamp(u, -limit, limit)."""
+    limit: float
+    slope: float = 1.702
+    shift: float = 1.0
+
+    def __post_init__(self):
+        if not self.limit > 0:
+            raise KernelError(f"a clamped unit's limit must be positive, got {self.limit}")
+
+
+def _expert_shapes(h, w_up, w_down, ids, wts, gated, what: str):
+    T, D = h.shape
+    E, F = w_down.shape[0], w_down.shape[2]
+    K = ids.shape[1]
+    up_rows = 2 * F if gated else F
+    if (tuple(w_up.shape) != (E, up_rows, D) or tuple(w_down.shape) != (E, D, F) or tuple(ids.shape) != (T, K) or tuple(wts.shape) != (T, K)
+            or not (w_up.is_contiguous() and w_down.is_contiguous() and ids.is_contiguous() and wts.is_contiguous())):
+        raise KernelError(f"{what}: h {tuple(h.shape)}, w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)}, ids "
+                          f"{tuple(ids.shape)} do not fit ({'gate and up rows stacked' if gated else 'experts without a gate'})")
+    return T, D, E, F, K
+
+
+def gated_unit(gu: torch.Tensor, unit: ClampedUnit, row_scale: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """gu [T, 2 F] (gate columns, then up columns) -> [T, F] in gu's type: the clamped unit of every pair, times
+    row_scale[t] (float32) when given, rounded once."""
+    require_gpu()
+    _dev(gu, "gu", dims=2)
+    T, F2 = gu.shape
+    if F2 % 2 or gu.dtype not in _DT:
+        raise KernelError(f"gated_unit: gate and up columns side by side, got {tuple(gu.shape)} {gu.dtype}")
+    if row_scale is not None:
+        _dev(row_scale, "row_scale", torch.float32, 1)
+        if row_scale.numel() != T or not row_scale.is_contiguous():
+            raise KernelError("gated_unit: one factor per row")
+    out = torch.empty((T, F2 // 2), dtype=gu.dtype, device=gu.device)
+    if T:
+        _check(_fn("moe", "bn_gated_unit")(_code(gu.dtype), out.data_ptr(), gu.data_ptr(), _rows(gu, "gu"),
+                                           row_scale.data_ptr() if row_scale is not None else None, T, F2 // 2,
+                                           float(unit.limit), float(unit.slope), float(unit.shift), _stream()), "gated_unit")
+    return out
 
 
 def moe_experts(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
-                activation: str = "relu2", weight_on_input: bool = True) -> PartialSums:
+                activation: str = "relu2", weight_on_input: bool = True, *, gated: Optional[ClampedUnit] = None,
+                extra_slabs: int = 0) -> PartialSums:
     """The chosen experts' outputs, expert e being w_down[e] act(w_up[e] x) (w_up [E, F, D], w_down [E, D, F], act one of
-    UNARY_ACTIVATIONS): slab j of the result [top_k, T, D] (float32) holds every token's j-th choice, computed on w h
-    (weight_on_input) or scaled by w afterwards.  The feed-forward's output is the sum of the slabs."""
+    UNARY_ACTIVATIONS), or, with `gated`, w_down[e] unit(gate rows . x, up rows . x) (w_up [E, 2 F, D]: F gate rows, then F
+    up rows): slab j of the result [top_k, T, D] (float32) holds every token's j-th choice, computed on w h
+    (weight_on_input) or scaled by w afterwards.  The feed-forward's output is the sum of the slabs.  extra_slabs: that
+    many more slabs behind the experts', left for the caller to fill."""
     require_gpu()
     _dev(h, "h", dims=2)
     _dev(w_up, "w_up", h.dtype, 3)
     _dev(w_down, "w_down", h.dtype, 3)
     _dev(ids, "ids", torch.int32, 2)
     _dev(wts, "wts", torch.float32, 2)
-    T, D = h.shape
-    E, F, _ = w_up.shape
-    K = ids.shape[1]
-    if (tuple(w_up.shape) != (E, F, D) or tuple(w_down.shape) != (E, D, F) or tuple(ids.shape) != (T, K) or tuple(wts.shape) != (T, K)
-            or not (w_up.is_contiguous() and w_down.is_contiguous() and ids.is_contiguous() and wts.is_contiguous())):
-        raise KernelError(f"moe_experts: h {tuple(h.shape)}, w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)}, ids "
-                          f"{tuple(ids.shape)} do not fit")
-    if activation not in UNARY_ACTIVATIONS:
+    T, D, E, F, K = _expert_shapes(h, w_up, w_down, ids, wts, gated is not None, "moe_experts")
+    if gated is None and activation not in UNARY_ACTIVATIONS:
         raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
     if max(D, F) > 16384 or K > 65535:
         raise KernelError(f"moe_experts: width {D} / expert width {F} above 16,384 values")
-    y = torch.empty((K, T, D), dtype=torch.float32, device=h.device)
+    y = torch.empty((K + int(extra_slabs), T, D), dtype=torch.float32, device=h.device)
+    unit = gated or ClampedUnit(1.0)
     run = 65535 // K                                      # tokens of one launch: a pair a row of the grid
     ld = _rows(h, "h")
     for t0 in range(0, T, run):
@@ -1910,7 +2054,9 @@ def moe_experts(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: 
         _check(_fn("moe", "bn_moe_experts")(_code(h.dtype), h.data_ptr() + t0 * ld * h.element_size(), ld, w_up.data_ptr(),
                                             w_down.data_ptr(), ids.data_ptr() + t0 * K * 4, wts.data_ptr() + t0 * K * 4,
                                             y.data_ptr() + t0 * D * 4, hidden.data_ptr(), n, T, D, F, K,
-                                            UNARY_ACTIVATIONS[activation], int(bool(weight_on_input)), _stream()), "moe_experts")
+                                            0 if gated is not None else UNARY_ACTIVATIONS[activation], int(bool(weight_on_input)),
+                                            int(gated is not None), float(unit.limit), float(unit.slope), float(unit.shift),
+                                            _stream()), "moe_experts")
     return PartialSums(y)
 
 
@@ -1925,32 +2071,28 @@ def moe_grouped_supported(T: int, D: int, F: int, dtype) -> bool:
 
 
 def moe_experts_grouped(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor, wts: torch.Tensor,
-                        activation: str = "relu2", weight_on_input: bool = True) -> PartialSums:
+                        activation: str = "relu2", weight_on_input: bool = True, *, gated: Optional[ClampedUnit] = None,
+                        extra_slabs: int = 0) -> PartialSums:
     """What moe_experts computes, for bf16 steps of many rows: the (token, choice) pairs are ordered by expert on the
     device and cut into tiles of up to MOE_TILE_ROWS rows of one expert, the inputs are gathered in that order (scaled
     and rounded there when the weight multiplies the input), and both products run as grouped matrix products on the matrix
     cores (the tiled kernel of gemm_mfma with a list of tiles).  Nothing comes back to the host; the launches' sizes depend
-    on the step's shape alone."""
+    on the step's shape alone.  gated, extra_slabs: as moe_experts's; the gate and up rows of an expert run as one grouped
+    product and the unit follows in a kernel of its own."""
     require_gpu()
     _dev(h, "h", torch.bfloat16, 2)
     _dev(w_up, "w_up", torch.bfloat16, 3)
     _dev(w_down, "w_down", torch.bfloat16, 3)
     _dev(ids, "ids", torch.int32, 2)
     _dev(wts, "wts", torch.float32, 2)
-    T, D = h.shape
-    E, F, _ = w_up.shape
-    K = ids.shape[1]
-    if (tuple(w_up.shape) != (E, F, D) or tuple(w_down.shape) != (E, D, F) or tuple(ids.shape) != (T, K) or tuple(wts.shape) != (T, K)
-            or not (w_up.is_contiguous() and w_down.is_contiguous() and ids.is_contiguous() and wts.is_contiguous())):
-        raise KernelError(f"moe_experts_grouped: h {tuple(h.shape)}, w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)}, ids "
-                          f"{tuple(ids.shape)} do not fit")
-    if activation not in UNARY_ACTIVATIONS:
+    T, D, E, F, K = _expert_shapes(h, w_up, w_down, ids, wts, gated is not None, "moe_experts_grouped")
+    if gated is None and activation not in UNARY_ACTIVATIONS:
         raise KernelError(f"unknown activation {activation!r}; known: {sorted(UNARY_ACTIVATIONS)}")
     ld = _rows(h, "h")
     if D % 8 or F % 8 or E > MOE_MAX_EXPERTS or ld % 8 or (h.data_ptr() | w_up.data_ptr() | w_down.data_ptr()) % 16:
         raise KernelError(f"moe_experts_grouped: widths {D} and {F} must be multiples of 8, rows 16-byte aligned, at most "
                           f"{MOE_MAX_EXPERTS} experts")
-    y = torch.empty((K, T, D), dtype=torch.float32, device=h.device)
+    y = torch.empty((K + int(extra_slabs), T, D), dtype=torch.float32, device=h.device)
     if T == 0:
         return PartialSums(y)
     n = T * K
@@ -1958,15 +2100,20 @@ def moe_experts_grouped(h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tenso
     work = torch.empty((2 * n + 3 * max_tiles + 1,), dtype=torch.int32, device=h.device)
     row_scale = torch.empty((n,), dtype=torch.float32, device=h.device)
     xg = torch.empty((n, D), dtype=torch.bfloat16, device=h.device)
-    hidden = torch.empty((n, F), dtype=torch.bfloat16, device=h.device)
+    hidden = torch.empty((n, 2 * F if gated is not None else F), dtype=torch.bfloat16, device=h.device)
     _check(_fn("moe", "bn_moe_group")(h.data_ptr(), ld, ids.data_ptr(), wts.data_ptr(), work.data_ptr(), row_scale.data_ptr(),
                                       xg.data_ptr(), T, D, E, K, MOE_TILE_ROWS, int(bool(weight_on_input)), _stream()),
            "moe_group")
     row_map, tiles = work.data_ptr() + 4 * n, work.data_ptr() + 8 * n
     n_tiles = tiles + 12 * max_tiles
     grouped = _fn("gemm_mfma", "bn_gemm_mfma_grouped")
-    _check(grouped(_code(torch.bfloat16), xg.data_ptr(), w_up.data_ptr(), hidden.data_ptr(), tiles, n_tiles, max_tiles, None, None,
-                   F * D, UNARY_ACTIVATIONS[activation], n, F, D, D, D, F, _stream()), "moe_experts_grouped(up)")
+    if gated is not None:
+        _check(grouped(_code(torch.bfloat16), xg.data_ptr(), w_up.data_ptr(), hidden.data_ptr(), tiles, n_tiles, max_tiles, None, None,
+                       2 * F * D, -1, n, 2 * F, D, D, D, 2 * F, _stream()), "moe_experts_grouped(gate and up)")
+        hidden = gated_unit(hidden, gated)
+    else:
+        _check(grouped(_code(torch.bfloat16), xg.data_ptr(), w_up.data_ptr(), hidden.data_ptr(), tiles, n_tiles, max_tiles, None, None,
+                       F * D, UNARY_ACTIVATIONS[activation], n, F, D, D, D, F, _stream()), "moe_experts_grouped(up)")
     _check(grouped(_code(torch.float32), hidden.data_ptr(), w_down.data_ptr(), y.data_ptr(), tiles, n_tiles, max_tiles, row_map,
                    None if weight_on_input else row_scale.data_ptr(), D * F, -1, n, D, F, F, F, D, _stream()),
            "moe_experts_grouped(down)")

@@ -25,6 +25,8 @@ split-half or in neighbouring pairs, over the first rope_dims dimensions) and ta
   distance_bias  tensors dist_a, dist_b [heads]: dist_a[h] * ln(1 + dist_b[h] * (i - j)) is taken off the score of
                  query i and key j
   sink           the softmax has one more term of score 0 and no value: p_j = exp(s_j) / (1 + sum exp(s))
+  value_is_key   there is no value projection: kv head g's value is its key projection as projected, before the key's norm
+                 and rotation (the tensor wv does not exist; the value heads are as wide as the key heads)
 """
 from __future__ import annotations
 
@@ -47,7 +49,7 @@ class Attention(Part):
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  position: PartSpec, window: int = 0, bias: bool = False, v_head_dim: int = 0,
                  qk_norm_eps: float | None = None, q_temp_coef: float = 0.0, q_temp_every: int = 0,
-                 distance_bias: bool = False, sink: bool = False, qk_norm_span: str = "head"):
+                 distance_bias: bool = False, sink: bool = False, qk_norm_span: str = "head", value_is_key: bool = False):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
         if head_dim % 2 or head_dim < 2 or head_dim > ops.MAX_HEAD_DIM:
@@ -58,6 +60,9 @@ class Attention(Part):
         self.position = POSITION_ENCODINGS.build(position)
         self.qkv, self.o = Linear(), Linear()
         self.vd = int(v_head_dim) or self.hs
+        self.value_is_key = bool(value_is_key)
+        if self.value_is_key and self.vd != self.hs:
+            raise ValueError(f"attention: values that are the keys are as wide as the keys, got {self.vd} and {self.hs}")
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.q_temp_coef, self.q_temp_every = float(q_temp_coef), int(q_temp_every)
         self.distance_bias, self.sink = bool(distance_bias), bool(sink)
@@ -67,13 +72,14 @@ class Attention(Part):
         if self.norm_projection and self.qk_norm_eps is None:
             raise ValueError("attention: a norm over the whole projection needs qk_norm_eps")
         self.general = (self.vd != self.hs or self.qk_norm_eps is not None or self.q_temp_every > 0
-                        or self.distance_bias or self.sink or getattr(self.position, "interleaved", False))
+                        or self.distance_bias or self.sink or getattr(self.position, "interleaved", False)
+                        or self.value_is_key)
         if self.general:
             if self.vd % 2 or self.vd < 2 or self.vd > ops.MAX_HEAD_DIM:
                 raise ValueError(f"attention: v_head_dim {self.vd} is not supported by the kernels (even, at most {ops.MAX_HEAD_DIM})")
             if self.has_bias:
                 raise ValueError("attention: head norms, a query temperature, a distance bias, a sink, a rotation in neighbouring "
-                                 "pairs or values of another width come without projection biases")
+                                 "pairs, values of another width or values that are the keys come without projection biases")
             self.takes_deferred_norm = self.gives_lazy_delta = False
         self.q_norm = self.k_norm = self.dist_a = self.dist_b = None
 
@@ -88,6 +94,8 @@ class Attention(Part):
     def tensors(self):
         t = {"wq": ParamSpec((self.q_dim, self.hidden)), "wk": ParamSpec((self.kv_dim, self.hidden)),
              "wv": ParamSpec((self.Hkv * self.vd, self.hidden)), "wo": ParamSpec((self.hidden, self.H * self.vd))}
+        if self.value_is_key:
+            del t["wv"]
         if self.qk_norm_eps is not None:
             nq, nk = (self.q_dim, self.kv_dim) if self.norm_projection else (self.hs, self.hs)
             t.update({"q_norm": ParamSpec((nq,), "ones"), "k_norm": ParamSpec((nk,), "ones")})
@@ -100,7 +108,8 @@ class Attention(Part):
 
     def load(self, tensors, device, dtype):
         # stacked on the device: the host holds no copy beside the file's own bytes
-        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wq", "wk", "wv")], dim=0).contiguous()
+        stacked = ("wq", "wk") if self.value_is_key else ("wq", "wk", "wv")
+        w = torch.cat([upload(tensors[n], device, dtype) for n in stacked], dim=0).contiguous()
         b = None
         if self.has_bias:
             b = torch.cat([upload(tensors[n], device, torch.float32) for n in ("bq", "bk", "bv")])
@@ -137,7 +146,7 @@ class Attention(Part):
         H, Hkv, hs, vd = self.H, self.Hkv, self.hs, self.vd
         if isinstance(h, ops.DeferredNorm):
             h = h.materialize()
-        width = H * hs + Hkv * (hs + vd)
+        width = H * hs + Hkv * (hs if self.value_is_key else hs + vd)
         if kv.writes:
             qkv = self.qkv(h)
         else:
@@ -149,7 +158,7 @@ class Attention(Part):
                           rope_dims=self.position.rope_dims, rope_interleaved=getattr(self.position, "interleaved", False),
                           seq_index=ctx.seq_index if kv.writes else None, block_table=kv.block_table if kv.writes else None,
                           k_pages=kv.k_pages if kv.writes else None, v_pages=kv.v_pages if kv.writes else None,
-                          v_transposed=True)
+                          v_transposed=True, v_from_k=self.value_is_key)
         out = torch.empty((h.shape[0], H * vd), dtype=h.dtype, device=h.device)
         bias = (self.dist_a, self.dist_b) if self.distance_bias else None
         on_matrix_cores = (ops.attention_general_supported(h.dtype, hs, vd) and ops.GENERAL_PROMPT_ON_MATRIX_CORES

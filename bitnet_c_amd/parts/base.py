@@ -243,6 +243,11 @@ class ResidualStream:
                 from .. import ops
                 p, self.pending = self.pending, None
                 return ops.add_normed_rmsnorm(self.x, p.delta, p.norm.weight, p.norm.eps, norm.weight, norm.eps, out_dtype)
+            if rows is None and getattr(norm, "passes_rows", False):
+                # no norm in front of the next part: the held-back output's norm, the sum, and the new rows handed on
+                from .. import ops
+                p, self.pending = self.pending, None
+                return ops.add_normed_rmsnorm(self.x, p.delta, p.norm.weight, p.norm.eps, out_dtype=out_dtype, rows_out=True)
             self.flush()
         if (rows is None and isinstance(self.pending, LazyDelta) and getattr(consumer, "takes_deferred_norm", False)
                 and getattr(norm, "deferrable", False)):

@@ -2,7 +2,10 @@
 (src/transformer/rmsnorm_scalar.c:4-13).  Computed in float32 whatever the activation
 type; the weight is kept in float32.  `scalar`: the model folder holds one number for all
 coordinates (a tensor without dimensions); it is spread over the coordinates at load, and
-every kernel that takes this norm, folded into a product or not, sees a weight vector."""
+every kernel that takes this norm, folded into a product or not, sees a weight vector.
+
+"none": no norm at all: the part behind it reads the stream itself, in the activations' type (a block whose norms sit on
+its parts' outputs only)."""
 from __future__ import annotations
 
 import torch
@@ -32,3 +35,23 @@ class RMSNorm(Part):
 
     def apply(self, x, delta, out_dtype, rows=None):
         return ops.add_rmsnorm(x, delta, self.weight, self.eps, out_dtype, rows)
+
+
+@NORMS.register("none")
+class NoNorm(Part):
+    """The stream as it is.  A held-back output that has a norm of its own is added by the same kernel that hands the
+    rows on (ResidualStream.normed)."""
+    prompt_capturable = True
+    passes_rows = True           # ResidualStream: no weight, no factor: the rows themselves
+
+    def __init__(self, dim: int = 0):
+        self.dim = int(dim)
+
+    def apply(self, x, delta, out_dtype, rows=None):
+        if rows is not None:
+            if delta is not None:
+                raise ValueError("a choice of rows leaves the stream as it is")
+            return ops.gather_rows(x, rows, out_dtype)
+        if delta is not None:
+            ops.residual_add(x, delta)
+        return ops.stream_rows(x, out_dtype)

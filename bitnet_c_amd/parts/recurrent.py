@@ -16,6 +16,11 @@ input (zero before the first token; the last h of a step is part of the state):
 "mingru": a gated recurrence whose gates read the current token alone:
     z = sigmoid(W_z h + b_z);  c = W_x h + b_x;  cand = c + 1/2 where c >= 0, sigmoid(c) below
     S <- (1 - z) S + z cand   element by element;   y = W_o (S * silu(W_g h))
+
+"lightning": linear attention with a matrix state per head and a decay that is a constant of the head (csrc/lightning.hip):
+    q, k = silu(W_q h), silu(W_k h)   heads x head_dim;   v = silu(W_v h)   heads x v_head_dim
+    S <- decay_head S + k_t v_t^T;    o_t = S^T q_t                       no other scale
+    y = W_o (o / rms_row(o) * norm * sigmoid(W_g h))                     the heads' outputs normed together, eps inside the root
 """
 from __future__ import annotations
 
@@ -124,4 +129,62 @@ class MinGRU(Part):
     def forward(self, h, ctx, kv):
         zxg = self.zxg(h)
         y = ops.mingru_scan(zxg, self.bz, self.bx, kv.state, ctx.slot_ids, self.W, **_sequences(ctx))
+        return self.o(y)
+
+
+@MIXERS.register("lightning")
+class Lightning(Part):
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+
+    def __init__(self, hidden: int, n_heads: int, head_dim: int, decay, eps: float, v_head_dim: int = 0,
+                 gate_activation: str = "sigmoid"):
+        self.hidden, self.H, self.hs, self.eps = int(hidden), int(n_heads), int(head_dim), float(eps)
+        self.vd = int(v_head_dim) or self.hs
+        self.decay_values = tuple(float(d) for d in decay)
+        if len(self.decay_values) != self.H or not all(0.0 <= d <= 1.0 for d in self.decay_values):
+            raise ValueError(f"lightning: one decay in [0, 1] per head, got {len(self.decay_values)} for {self.H} heads")
+        if not ops.lightning_supported(self.hs, self.vd):
+            raise ValueError(f"lightning: head_dim {self.hs} is not supported by the kernel (at most {ops.LIGHTNING_MAX_DIM})")
+        if gate_activation not in ops.UNARY_ACTIVATIONS:
+            raise ValueError(f"lightning: unknown gate activation {gate_activation!r}; known: {sorted(ops.UNARY_ACTIVATIONS)}")
+        self.gate_activation = gate_activation
+        self.qkvg, self.o = Linear(), Linear()        # the four projections stacked: one product
+        self.decay = self.norm = None
+
+    @property
+    def k_col(self):
+        return self.H * self.hs
+
+    @property
+    def v_col(self):
+        return 2 * self.H * self.hs
+
+    @property
+    def g_col(self):
+        return 2 * self.H * self.hs + self.H * self.vd
+
+    def tensors(self):
+        D, A, B = self.hidden, self.H * self.hs, self.H * self.vd
+        return {"wq": ParamSpec((A, D)), "wk": ParamSpec((A, D)), "wv": ParamSpec((B, D)), "wg": ParamSpec((B, D)),
+                "norm": ParamSpec((B,), "ones"), "wo": ParamSpec((D, B))}
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wq", "wk", "wv", "wg")], dim=0).contiguous()
+        self.qkvg.load(w, None, device, dtype)
+        self.o.load(tensors["wo"], None, device, dtype)
+        self.norm = upload(tensors["norm"], device, torch.float32)
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float64).to(torch.float32).to(device)
+
+    def linears(self):
+        return [self.qkvg, self.o]
+
+    def cache_need(self) -> CacheNeed:
+        # per head a [head_dim, v_head_dim] matrix, float32
+        return CacheNeed(state=StateNeed((self.H * self.hs * self.vd,), torch.float32, device_addressed=True))
+
+    def forward(self, h, ctx, kv):
+        x = self.qkvg(h)
+        o = ops.lightning_scan(x, 0, self.k_col, self.v_col, self.decay, kv.state, ctx.slot_ids, self.H, self.hs, self.vd,
+                               **_sequences(ctx))
+        y = ops.row_norm_gate(o, x[:, self.g_col:], self.norm, self.eps, self.gate_activation)
         return self.o(y)
