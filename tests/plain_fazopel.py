@@ -84,6 +84,18 @@ def rotate_halves(x: torch.Tensor, positions, rot: dict, angle_dtype=F64) -> tor
 
 # ---- mixers ----------------------------------------------------------------------------------------------------
 
+def decayed_sums(q, k, v, decay, state=None):
+    """q, k [T, H, d], v [T, H, vd], decay [H]: token by token S <- decay S + k v^T, o = S^T q.  Returns (o [T, H, vd],
+    the state after the last token [H, d, vd])."""
+    T, H, d = q.shape
+    S = torch.zeros((H, d, v.shape[-1]), dtype=F64) if state is None else state.clone()
+    o = torch.zeros((T, H, v.shape[-1]), dtype=F64)
+    for t in range(T):
+        S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    return o, S
+
+
 def lightning(h, W, p, m, eps, state=None):
     """Linear attention with a fixed decay per head.  q, k = silu of their projections [heads, dim], v = silu of its
     projection [heads, vdim]; per head S <- decay S + k v^T, o = S^T q; the heads' outputs side by side are divided by
@@ -94,12 +106,7 @@ def lightning(h, W, p, m, eps, state=None):
     q = silu(h @ W[p + "q"].T).reshape(T, H, d)
     k = silu(h @ W[p + "k"].T).reshape(T, H, d)
     v = silu(h @ W[p + "v"].T).reshape(T, H, vd)
-    decay = torch.tensor([float(x) for x in m["decay"]], dtype=F64)
-    S = torch.zeros((H, d, vd), dtype=F64) if state is None else state.clone()
-    o = torch.zeros((T, H, vd), dtype=F64)
-    for t in range(T):
-        S = decay[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
-        o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+    o, S = decayed_sums(q, k, v, torch.tensor([float(x) for x in m["decay"]], dtype=F64), state)
     y = unit_rms(o.reshape(T, H * vd), eps) * W[p + "norm"] * sigmoid(h @ W[p + "g"].T)
     return y @ W[p + "o"].T, S
 
@@ -151,30 +158,42 @@ def expert_unit(h, W, p, limit: float):
     return (g * sigmoid(GATE_SLOPE * g) * (u + 1.0)) @ W[p + "down"].T
 
 
-def route(h, W, p, mlp, router_input=None):
+def route(h, W, p, mlp, margins=None):
     """(chosen experts [T, top], their weights [T, top]).  Scores are the softmax of the router's logits over all
     experts; the choice goes by score + correction, the weights are the plain scores of the chosen, divided by their sum
-    and multiplied by router.scale."""
+    and multiplied by router.scale.  margins: a list that receives, per token, how far the last chosen expert's choice
+    score lies above the first one left out, in units of what a small relative change of the logits does to a score
+    (score times the logits' root mean square): a small number is a close call."""
     r = mlp["router"]
-    x = h if router_input is None else router_input
-    z = x @ W[p + "router"].T
+    z = h @ W[p + "router"].T
     e = torch.exp(z - z.max(dim=-1, keepdim=True).values)
     s = e / e.sum(dim=-1, keepdim=True)
-    chosen = torch.topk(s + W[p + "correction"], r["top"], dim=-1).indices
+    c = s + W[p + "correction"]
+    chosen = torch.topk(c, r["top"], dim=-1).indices
+    if margins is not None:
+        if r["top"] < r["experts"]:
+            order = torch.argsort(c, dim=-1, descending=True)
+            last, nxt = order[:, r["top"] - 1:r["top"]], order[:, r["top"]:r["top"] + 1]
+            gap = (torch.gather(c, 1, last) - torch.gather(c, 1, nxt))[:, 0]
+            size = torch.maximum(torch.gather(s, 1, last), torch.gather(s, 1, nxt))[:, 0] * z.pow(2).mean(dim=-1).sqrt()
+            margins.append(gap / size.clamp_min(1e-300))
+        else:
+            margins.append(torch.full((h.shape[0],), float("inf"), dtype=F64))
     w = torch.gather(s, 1, chosen)
-    w = w / (w.sum(dim=-1, keepdim=True) + WEIGHT_FLOOR) * r["scale"]
+    w = w / (w.sum(dim=-1, keepdim=True) + WEIGHT_FLOOR) * r.get("scale", 1.0)
     return chosen, w
 
 
-def moe_ff(h, W, p, mlp):
+def moe_ff(h, W, p, mlp, margins=None):
     """The weighted sum of the chosen experts, plus (when the layer has one) a shared expert that every token runs,
     times sigmoid(W_sg h)."""
-    chosen, w = route(h, W, p, mlp)
+    chosen, w = route(h, W, p, mlp, margins)
     out = torch.zeros_like(h)
-    for t in range(h.shape[0]):
-        for j in range(chosen.shape[1]):
-            e = int(chosen[t, j])
-            out[t] += w[t, j] * expert_unit(h[t:t + 1], W, f"{p}e{e}.", mlp["expert"]["limit"])[0]
+    for e in range(mlp["router"]["experts"]):               # expert by expert: the tokens that chose it, with their weights
+        share = (w * (chosen == e)).sum(dim=-1)
+        rows = torch.nonzero((chosen == e).any(dim=-1))[:, 0]
+        if rows.numel():
+            out[rows] += share[rows, None] * expert_unit(h[rows], W, f"{p}e{e}.", mlp["expert"]["limit"])
     if mlp.get("shared"):
         out = out + sigmoid(h @ W[p + "shared.sg"].T) * expert_unit(h, W, p + "shared.", mlp["shared"]["limit"])
     return out
@@ -187,7 +206,7 @@ def weights_prefix(c: dict, i: int) -> str:
     return f"l{c['layers'][i].get('weights_of', i)}."
 
 
-def layer_forward(c, W, i, x, angle_dtype=F64, round_to=None, carry=None, pos0: int = 0):
+def layer_forward(c, W, i, x, angle_dtype=F64, round_to=None, carry=None, pos0: int = 0, margins=None):
     """x <- x + norm1(mixer(x)); x <- x + norm2(ff(x)): the sublayers read x itself, the norms sit on their outputs.
     carry: what the layer keeps from earlier tokens (a state or keys and values).  Returns (x, carry after)."""
     L, eps, p = c["layers"][i], c["norm"]["eps"], weights_prefix(c, i)
@@ -203,19 +222,24 @@ def layer_forward(c, W, i, x, angle_dtype=F64, round_to=None, carry=None, pos0: 
     mlp = L.get("mlp")
     if mlp is not None:
         h = rd(x)
-        y = dense_ff(h, W, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, W, p + "mlp.", mlp)
+        y = dense_ff(h, W, p + "mlp.") if mlp["kind"] == "dense" else moe_ff(h, W, p + "mlp.", mlp, margins)
         x = x + unit_rms(y, eps) * W[p + "norm2"]
     return x, carry
 
 
-def forward(c: dict, W: dict, tokens, angle_dtype=F64, round_to=None, layers_out=None) -> torch.Tensor:
+def forward(c: dict, W: dict, tokens, layers_out=None, angle_dtype=F64, round_to=None, margins=None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  round_to: the stream is rounded to this type where a sublayer reads it
-    (what an engine with activations of that type does); layers_out: a list that receives the stream after every layer."""
+    (what an engine with activations of that type does); layers_out: a list that receives the stream after every layer;
+    margins: a list that receives, per token, the smallest routing margin over all layers (see route)."""
     x = W["embed"][torch.as_tensor(list(tokens), dtype=torch.long)]
+    per_layer = [] if margins is not None else None
     for i in range(len(c["layers"])):
-        x, _ = layer_forward(c, W, i, x, angle_dtype, round_to)
+        x, _ = layer_forward(c, W, i, x, angle_dtype, round_to, margins=per_layer)
         if layers_out is not None:
             layers_out.append(x.clone())
+    if margins is not None:
+        low = torch.stack(per_layer).min(dim=0).values if per_layer else torch.full((len(tokens),), float("inf"), dtype=F64)
+        margins.extend(low.tolist())
     h = unit_rms(x, c["norm"]["eps"]) * W["final.norm"]
     if round_to is not None:
         h = h.to(round_to).to(F64)
@@ -226,5 +250,5 @@ def generate(c: dict, W: dict, prompt, n_new: int, angle_dtype=F64, round_to=Non
     """Greedy continuation, the whole sequence run again for every token."""
     seq = list(prompt)
     for _ in range(n_new):
-        seq.append(int(forward(c, W, seq, angle_dtype, round_to)[-1].argmax()))
+        seq.append(int(forward(c, W, seq, angle_dtype=angle_dtype, round_to=round_to)[-1].argmax()))
     return seq[len(prompt):]
