@@ -211,11 +211,35 @@ def _sonodra_configs(z):
     return son, _llama_config(z)
 
 
+def _fazopel_configs(z):
+    """(Fazopel config.json, Sonodra config.json, Llama config.json) of equal width, layers and attention heads: two
+    lightning layers (heads as many and as wide as the attention's), then an attention layer, repeated; the first layer's
+    feed-forward is the dense one, the others choose `top` of `experts` gated experts beside a shared expert of an
+    expert's width, so that the three matrices of the units a token runs are as large as the gated feed-forward's three."""
+    gated = _llama_config(z)["intermediate_size"]
+    ff = gated // (z["top"] + 1) // 64 * 64
+    moe = dict(kind="moe", expert=dict(ff=ff, limit=7.0), router=dict(experts=z["experts"], top=z["top"], scale=2.5),
+               shared=dict(ff=ff, limit=7.0))
+    H = z["heads"]
+    lin = dict(heads=H, dim=z["dim"], vdim=z["dim"], decay=[round(1.0 - 2.0 ** -(5.0 + 3.0 * h / max(H - 1, 1)), 9) for h in range(H)])
+    att = dict(heads=H, kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=z["dim"] ** -0.5,
+               rot=dict(base=500000.0, dims=z["rot_dims"], scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+    layers = []
+    for i in range(z["layers"]):
+        mlp = dict(kind="dense", ff=z["ff"]) if i == 0 else moe
+        layers.append(dict(type="attention", mixer=att, mlp=mlp) if i % 3 == 2 else dict(type="lightning", mixer=lin, mlp=mlp))
+    faz = dict(architecture="Fazopel", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-6), layers=layers)
+    return (faz,) + _sonodra_configs(z)
+
+
 def _design_configs(design, z):
-    """(the design's config.json, Llama config.json) of equal width, layers, attention heads and (nearly) equal weight bytes."""
+    """name -> config.json: the design, then what it is measured beside (the Llama-style decoder of equal width, layers,
+    attention heads and (nearly) equal weight bytes read per token; for Fazopel also Sonodra, the closest of the others)."""
+    if design == "fazopel":
+        return dict(zip(("fazopel", "sonodra", "llama"), _fazopel_configs(z)))
     if design == "sonodra":
-        return _sonodra_configs(z)
-    return _sunusun_configs(z)
+        return dict(zip(("sonodra", "llama"), _sonodra_configs(z)))
+    return dict(zip(("sunusun", "llama"), _sunusun_configs(z)))
 
 
 def _sunusun_configs(z):
@@ -246,7 +270,9 @@ def bench_design(args) -> int:
     PREFILL, lens = args.prefill_tokens, (256, 1024)
     out = {"design": args.design, "size": args.design_size, "sizes": z, "dtype": "bf16", "steps": args.steps, "warmup": args.warmup,
            "prefill_tokens": PREFILL, "decode_prompt_lens": list(lens), "data": "synthetic: random N(0,0.02) weights, uniform token ids"}
-    for name, raw in zip((args.design, "llama"), _design_configs(args.design, z)):
+    for name, raw in _design_configs(args.design, z).items():
+        if args.design_alone and name != args.design:
+            continue
         arch = architecture_for(raw)
         cfg = arch.config_cls.from_dict(raw)
         plan = arch.build_plan(cfg)
@@ -321,7 +347,8 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=0, help="longest sequence (default: the shape's)")
     ap.add_argument("--prompt-lens", default=None, metavar="LO,HI", help="prompt lengths of the decode batches")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the measured prompt step")
-    ap.add_argument("--design", choices=["sunusun", "sonodra"], default=None,
+    ap.add_argument("--design-alone", action="store_true", help="with --design: the design alone, for profiling")
+    ap.add_argument("--design", choices=["sunusun", "sonodra", "fazopel"], default=None,
                     help="instead of the benchmark: prefill and decode of this design beside the Llama-style decoder of equal "
                          "width, heads, layers and weight bytes, at the sizes of --design-size (random weights; one JSON line)")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="2048")
