@@ -84,8 +84,10 @@ _SIGNATURES = {
     },
     "lightning": {
         "bn_lightning_supports": [c_int, c_int],
+        "bn_lightning_chunked": [c_int, c_int],
+        "bn_lightning_prefers_chunks": [c_int, c_int, c_int, c_int],
         "bn_lightning_scan": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
-                              c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+                              c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p],
         "bn_row_norm_gate": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_int, c_void_p],
     },
     "state_mixers": {
@@ -1781,13 +1783,21 @@ def lightning_supported(dk: int, dv: int) -> bool:
     return 1 <= dk <= LIGHTNING_MAX_DIM and dv >= 1
 
 
+def lightning_chunked(dk: int, dv: int) -> bool:
+    """Whether prompt steps of these head sizes take the chunked form of the recurrence."""
+    return bool(_fn("lightning", "bn_lightning_chunked")(int(dk), int(dv)))
+
+
 def lightning_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, decay: torch.Tensor, state: torch.Tensor, slot_ids,
-                   H: int, dk: int, dv: int, *, tiles=None, seq_lens=None) -> torch.Tensor:
+                   H: int, dk: int, dv: int, *, tiles=None, seq_lens=None, chain: Optional[bool] = None) -> torch.Tensor:
     """Linear attention with a fixed decay per head over every sequence of a step; float32 [T, H dv].  x [T, >= ...] in
     the activations' type holds the projections side by side: queries at column q_col and keys at k_col (H dk wide),
     values at v_col (H dv wide); each passes silu in float32.  decay [H] float32.  state [slots, >= H dk dv] float32, the
     heads' matrices [H][dk][dv], updated in place; a sequence at position 0 starts from zeros.  Per head, in float32:
-        S <- decay S + k_t v_t^T;  o_t = S^T q_t."""
+        S <- decay S + k_t v_t^T;  o_t = S^T q_t.
+    A prompt step (tiles) of a key width that lightning_chunked() takes can run the same sums chunk by chunk on the matrix
+    cores, in float32, instead of token by token as decode steps do.  chain: True the token-by-token kernel, False the
+    chunks where they can be, None whichever is the faster for this many sequences and heads."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(decay, "decay", torch.float32, 1)
@@ -1806,9 +1816,16 @@ def lightning_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, decay: t
         raise KernelError("lightning_scan: a decode step has one length per row")
     o = torch.empty((T, H * dv), dtype=torch.float32, device=x.device)
     if T and n_seqs:
+        prepared = None
+        if tiles is not None and chain is not True and lightning_chunked(dk, dv) and (
+                chain is False or _fn("lightning", "bn_lightning_prefers_chunks")(n_seqs, H, dk, dv)):
+            # the chunked form's own copy of the step's q, k and v: silu applied, float32, head by head
+            prepared = torch.empty(H * T * (2 * ((dk + 3) // 4 * 4) + (dv + 3) // 4 * 4), dtype=torch.float32, device=x.device)
         _check(_fn("lightning", "bn_lightning_scan")(_code(x.dtype), x.data_ptr(), ld, int(q_col), int(k_col), int(v_col),
                                                      decay.data_ptr(), o.data_ptr(), state.data_ptr(), stride, tl, n_seqs, sl,
-                                                     slot_ids.data_ptr(), H, dk, dv, _stream()), "lightning_scan")
+                                                     slot_ids.data_ptr(), H, dk, dv, T,
+                                                     prepared.data_ptr() if prepared is not None else None, _stream()),
+               "lightning_scan")
     return o
 
 

@@ -163,11 +163,13 @@ def test_head_norms_rotation_and_values_that_are_the_keys(dtype, H, G, hs, rd, s
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("chain", [False, True])
 @pytest.mark.parametrize("H,dk,dv", [(3, 16, 24), (2, 10, 70), (1, 64, 64), (2, 128, 130), (1, 200, 8), (5, 1, 1)])
-def test_the_decayed_sums_over_prompts_portions_and_single_tokens(dtype, H, dk, dv):
+def test_the_decayed_sums_over_prompts_portions_and_single_tokens(dtype, H, dk, dv, chain):
     """The recurrence over a step of three sequences of unequal lengths (one continues from a state, one starts in a row
     that a former sequence left its state in), then one token each, against the recurrence written token by token; the
-    projections lie side by side in one tensor with other columns between and around them."""
+    projections lie side by side in one tensor with other columns between and around them.  The prompt step in the form
+    the sizes choose (chunks on the matrix cores where the key width allows) and in the token-by-token form."""
     from bitnet_c_amd import ops
     g = torch.Generator().manual_seed(dk * 7 + dv)
     decay = torch.tensor([0.0, 1.0, 0.9, 0.999, 0.5][:H] if H <= 5 else [0.9] * H, dtype=torch.float64)
@@ -200,7 +202,7 @@ def test_the_decayed_sums_over_prompts_portions_and_single_tokens(dtype, H, dk, 
         r += n
     tiles.append([0, 0, 0, 0])                                 # a tile of no rows
     x = torch.cat([t[:-1] for t in xs]).to(DEV)
-    o = ops.lightning_scan(x, qc, kc, vc, decay.float().to(DEV), st, i32(slots), H, dk, dv, tiles=i32(tiles))
+    o = ops.lightning_scan(x, qc, kc, vc, decay.float().to(DEV), st, i32(slots), H, dk, dv, tiles=i32(tiles), chain=chain)
     tol = 2e-5 if dtype == torch.float32 else 1e-4            # the inputs are the same rounded numbers on both sides
     close_ = lambda a, b: rel_err(a, b) < tol
     assert close_(o, torch.cat([w[:-1] for w in want]).reshape(sum(lens), -1))
@@ -213,6 +215,66 @@ def test_the_decayed_sums_over_prompts_portions_and_single_tokens(dtype, H, dk, 
     for b in range(3):
         assert close_(st[slots[b], :H * dk * dv], S_after[b].reshape(-1))
     assert torch.equal(st[5], before[5]) and torch.equal(st[0], before[0]) and torch.equal(st[:, H * dk * dv:], before[:, H * dk * dv:])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H,dk,dv,seqs", [(2, 64, 64, 1), (2, 128, 128, 1), (3, 96, 40, 1), (1, 32, 16, 1), (20, 48, 64, 1),
+                                          (40, 64, 72, 1)])
+def test_the_chunked_form_at_the_edges_of_its_chunks(dtype, H, dk, dv, seqs):
+    """Prompt steps whose sequences end just before, at and just behind a chunk of 64 tokens and a block of 16, some
+    continuing from a state at a position that is no multiple of either; few heads and many, widths that are no multiple
+    of a tile's 16.  Against the recurrence written token by token, and the state left behind against both; then the same
+    step on the token-by-token kernel."""
+    from bitnet_c_amd import ops
+    assert ops.lightning_chunked(dk, dv)
+    g = torch.Generator().manual_seed(H * 1000 + dk + dv)
+    decay = torch.tensor([0.97, 0.5, 0.9995, 0.0, 1.0], dtype=torch.float64).repeat(H // 5 + 1)[:H]
+    lens = [63, 64, 65, 128, 129, 2, 200, 15, 16, 17, 1] * seqs
+    first = [0, 7, 0, 0, 70, 3, 0, 64, 0, 1, 9] * seqs
+    W = 2 * H * dk + H * dv + 8
+    qc, kc, vc = 0, H * dk, 2 * H * dk + 8
+    n_slots = len(lens) + 2
+    state = torch.zeros(n_slots, H * dk * dv, dtype=torch.float32)
+    slots = list(range(n_slots - 1, 1, -1))[:len(lens)]
+    xs, want, S_after = [], [], []
+
+    def halves(x):
+        x = x.double()
+        return (pf.silu(x[:, qc:qc + H * dk]).view(-1, H, dk), pf.silu(x[:, kc:kc + H * dk]).view(-1, H, dk),
+                pf.silu(x[:, vc:vc + H * dv]).view(-1, H, dv))
+    for b, (n, p0) in enumerate(zip(lens, first)):
+        S0 = None
+        if p0:
+            S0 = 0.5 * torch.randn(H, dk, dv, generator=g).float().double()
+            state[slots[b]] = S0.reshape(-1).float()
+        else:
+            state[slots[b]] = 3.0                              # a former owner's state: ignored at position 0
+        x = (0.7 * torch.randn(n, W, generator=g)).to(dtype)
+        o, S = pf.decayed_sums(*halves(x), decay, S0)
+        xs.append(x)
+        want.append(o.reshape(n, -1))
+        S_after.append(S.reshape(-1))
+    tiles, r = [], 0
+    for b, n in enumerate(lens):
+        tiles.append([b, r, n, first[b]])
+        r += n
+    x = torch.cat(xs).to(DEV)
+    want, S_after = torch.cat(want), torch.stack(S_after)
+    tol = 2e-5 if dtype == torch.float32 else 1e-4            # the inputs are the same rounded numbers on both sides
+    outs = []
+    for chain in (False, True):
+        st = state.to(DEV)
+        o = ops.lightning_scan(x, qc, kc, vc, decay.float().to(DEV), st, i32(slots), H, dk, dv, tiles=i32(tiles), chain=chain)
+        # sequence by sequence and head by head (each against its own size: a head that never decays grows far beyond
+        # the others): a short sequence is not hidden by a long one
+        for b in range(len(lens)):
+            rows = slice(tiles[b][1], tiles[b][1] + lens[b])
+            for h in range(H):
+                assert rel_err(o[rows, h * dv:(h + 1) * dv], want[rows, h * dv:(h + 1) * dv]) < tol, (chain, b, h)
+                assert rel_err(st[slots[b]].view(H, -1)[h], S_after[b].view(H, -1)[h]) < tol, (chain, b, h)
+        assert torch.equal(st[:2].cpu(), state[:2])            # rows of no sequence of the step
+        outs.append(o)
+    assert rel_err(outs[0], outs[1]) < 2 * tol
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
