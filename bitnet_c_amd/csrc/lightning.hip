@@ -14,9 +14,10 @@
 //                        chunks that all threads stage (silu applied) in shared memory, the waves walk a chunk token by
 //                        token and leave their partial sums, which are added in wave order.  The order of every sum is
 //                        a function of the sizes alone, so a token's output does not depend on how the step was cut.
-//                        This "chain" form serves decode steps and key widths above LC_MAX_DIM.
-//   the chunked form     prompt steps of key widths up to LC_MAX_DIM: a workgroup owns (sequence, head, 16 NCT value columns)
-//                        and takes the tokens in chunks of 64.  With d the decay, S the state before the chunk, n its tokens:
+//                        This "chain" form serves decode steps, key widths above LC_MAX_DIM and prompt steps of so
+//                        many sequences that it fills the chip (bn_lightning_prefers_chunks).
+//   the chunked form     other prompt steps: a workgroup owns (sequence, head, 16 value columns) and takes the tokens in
+//                        chunks of 64, from a float32 copy of silu(q), silu(k), silu(v) that a kernel in front makes.  With d the decay, S the state before the chunk, n its tokens:
 //                            A_ij = (q_i . k_j) d^(i-j) for j <= i,    o_i = sum_j A_ij v_j + d^(i+1) S^T q_i,
 //                            S   <- d^n S + sum_j d^(n-1-j) k_j v_j^T
 //                        which is the chain's sum in another order.  All four products run on the matrix cores in float32
