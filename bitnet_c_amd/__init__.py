@@ -9,10 +9,10 @@ Llama-style dense decoder, for Sunusun (recurrent and attention layers listed in
     out = llm.generate([[1, 2, 3], [4, 5]], max_new_tokens=16, temperature=0.0)
 """
 from .api import LLM, load  # noqa: F401
-from .config import FazopelConfig, LlamaConfig, SonodraConfig, SunusunConfig, load_config, register_architecture  # noqa: F401
+from .config import FazopelConfig, LlamaConfig, MutiraxConfig, SonodraConfig, SunusunConfig, load_config, register_architecture  # noqa: F401
 from .engine import Engine, Request, Result, StepEntry  # noqa: F401
 from .sampling import SamplingParams  # noqa: F401
 from .weights import WeightError, write_model_folder  # noqa: F401
 
-__all__ = ["LLM", "load", "Engine", "StepEntry", "Request", "Result", "SamplingParams", "LlamaConfig", "SunusunConfig", "SonodraConfig", "FazopelConfig",
+__all__ = ["LLM", "load", "Engine", "StepEntry", "Request", "Result", "SamplingParams", "LlamaConfig", "SunusunConfig", "SonodraConfig", "FazopelConfig", "MutiraxConfig",
            "load_config", "register_architecture", "WeightError", "write_model_folder"]

@@ -42,7 +42,8 @@ struct GenArgs {
     const float* dist_b;
     int q_stride, out_stride, bt_stride, H, Hkv;
     float scale;
-    int sink;
+    int sink;                 // 1: one more term without a value in the softmax's denominator, exp(sink_values[head])
+    const float* sink_values; // [H] float32, or null: the term's score is 0
     int window;               // 0: every earlier key; else the last `window` positions, the query's own included
 };
 
@@ -163,12 +164,13 @@ __global__ __launch_bounds__(AG_WAVES * BN_WAVE) void attn_general_prompt_kernel
             acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[t], pb, acc[t], 0, 0, 0);
         }
     }
-    // the sink: a term 2^(0 - m') with no value, m' = max(m, 0)
+    // the sink: a term 2^(sv - m') with no value, m' = max(m, sv)
     float fa = 1.f;
     if (a.sink) {
-        const float m2 = fmaxf(m, 0.f);
+        const float sv = a.sink_values ? a.sink_values[head] * AG_LOG2E : 0.f;       // the sink's score in the exponent's base 2
+        const float m2 = fmaxf(m, sv);
         fa = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m2);
-        l = fmaf(l, fa, __builtin_amdgcn_exp2f(-m2));
+        l = fmaf(l, fa, __builtin_amdgcn_exp2f(sv - m2));
     }
     const float inv = l > 0.f ? fa / l : 0.f;
     if (!col_ok) return;
@@ -198,6 +200,7 @@ struct GenDecodeArgs {
     float* part_ml;           // [n_seqs H, n_splits, 2]: maximum (natural exponent) and sum of the weights
     const int* max_len;       // != null: the longest sequence's key count; the keys per split follow from it
     int q_stride, out_stride, bt_stride, H, Hkv, n_splits, chunk, window, sink;
+    const float* sink_values; // [H] float32, or null (score 0)
     float scale;
 };
 
@@ -338,9 +341,10 @@ __global__ __launch_bounds__(BN_WAVE) void attn_general_decode_kernel(GenDecodeA
     }
     float fa = 1.f;
     if (a.sink) {
-        const float m2 = fmaxf(m, 0.f);
+        const float sv = a.sink_values ? a.sink_values[head] * AG_LOG2E : 0.f;       // the sink's score in the exponent's base 2
+        const float m2 = fmaxf(m, sv);
         fa = m == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m2);
-        l = fmaf(l, fa, __builtin_amdgcn_exp2f(-m2));
+        l = fmaf(l, fa, __builtin_amdgcn_exp2f(sv - m2));
     }
     const float inv = l > 0.f ? fa / l : 0.f;
     bf16* op = a.out + (size_t)seq * a.out_stride + (size_t)head * VD + 4 * g;
@@ -360,12 +364,14 @@ __global__ __launch_bounds__(BN_WAVE) void attn_general_decode_kernel(GenDecodeA
 __global__ __launch_bounds__(BN_WAVE) void attn_general_combine_kernel(bf16* __restrict__ out, int out_stride,
                                                                        const float* __restrict__ part_o,
                                                                        const float* __restrict__ part_ml, int H, int vd,
-                                                                       int n_splits, int sink) {
+                                                                       int n_splits, int sink,
+                                                                       const float* __restrict__ sink_values) {
     const int row = blockIdx.x, tok = row / H, head = row - tok * H;
     const float* ml = part_ml + (size_t)row * n_splits * 2;
-    float m = sink ? 0.f : -INFINITY;
+    const float sv = sink && sink_values ? sink_values[head] : 0.f;
+    float m = sink ? sv : -INFINITY;
     for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
-    float den = sink ? expf(-m) : 0.f;
+    float den = sink ? expf(sv - m) : 0.f;
     if (m != -INFINITY)
         for (int s = 0; s < n_splits; ++s) den = fmaf(expf(ml[2 * s] - m), ml[2 * s + 1], den);
     const float inv = den > 0.f ? 1.0f / den : 0.f;
@@ -407,7 +413,7 @@ static int ag_launch_dt(const GenArgs& a, int vd, dim3 grid, hipStream_t s) {
 extern "C" int bn_attn_general_prompt(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                                       const void* v_pages, const int* block_table, int bt_stride, const int* tiles, int n_tiles,
                                       int H, int Hkv, int hs, int vd, float scale, const float* dist_a, const float* dist_b,
-                                      int sink, int window, hipStream_t s) {
+                                      int sink, const float* sink_values, int window, hipStream_t s) {
     if (n_tiles <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || window < 0 || !bn_attn_general_supports(hs, vd)) return BN_ERR_ARG;
     if (!q || !out || !k_pages || !v_pages || !block_table || !tiles || (dist_a == nullptr) != (dist_b == nullptr)) return BN_ERR_ARG;
     if (q_stride % 8 || out_stride % 4 || (((uintptr_t)q | (uintptr_t)k_pages | (uintptr_t)v_pages) & 15) || ((uintptr_t)out & 7))
@@ -416,7 +422,7 @@ extern "C" int bn_attn_general_prompt(const void* q, int q_stride, void* out, in
     a.q = (const bf16*)q; a.out = (bf16*)out; a.k_pages = (const bf16*)k_pages; a.v_pages = (const bf16*)v_pages;
     a.block_table = block_table; a.tiles = tiles; a.dist_a = dist_a; a.dist_b = dist_b;
     a.q_stride = q_stride; a.out_stride = out_stride; a.bt_stride = bt_stride; a.H = H; a.Hkv = Hkv;
-    a.scale = scale; a.sink = sink ? 1 : 0; a.window = window;
+    a.scale = scale; a.sink = sink ? 1 : 0; a.sink_values = sink ? sink_values : nullptr; a.window = window;
     const dim3 grid(n_tiles, (H + AG_WAVES - 1) / AG_WAVES);
     switch (hs / 32) {
         case 1: return ag_launch_dt<1>(a, vd, grid, s);
@@ -448,7 +454,7 @@ static int ag_launch_decode_dt(const GenDecodeArgs& a, int vd, dim3 grid, hipStr
 extern "C" int bn_attn_general_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                                       const void* v_pages, const int* block_table, int bt_stride, const int* seq_lens, int n_seqs,
                                       int H, int Hkv, int hs, int vd, float scale, const float* dist_a, const float* dist_b,
-                                      int sink, int window, int n_splits, int chunk, float* part_o, float* part_ml,
+                                      int sink, const float* sink_values, int window, int n_splits, int chunk, float* part_o, float* part_ml,
                                       const int* max_len, hipStream_t s) {
     if (n_seqs <= 0 || H <= 0 || Hkv <= 0 || H % Hkv || window < 0 || n_splits < 1 || !bn_attn_general_supports(hs, vd)) return BN_ERR_ARG;
     if (!q || !out || !k_pages || !v_pages || !block_table || !seq_lens || (dist_a == nullptr) != (dist_b == nullptr)) return BN_ERR_ARG;
@@ -462,7 +468,7 @@ extern "C" int bn_attn_general_decode(const void* q, int q_stride, void* out, in
     a.block_table = block_table; a.seq_lens = seq_lens; a.dist_a = dist_a; a.dist_b = dist_b; a.part_o = part_o; a.part_ml = part_ml;
     a.max_len = n_splits > 1 ? max_len : nullptr;
     a.q_stride = q_stride; a.out_stride = out_stride; a.bt_stride = bt_stride; a.H = H; a.Hkv = Hkv; a.n_splits = n_splits;
-    a.chunk = chunk; a.window = window; a.sink = sink ? 1 : 0; a.scale = scale;
+    a.chunk = chunk; a.window = window; a.sink = sink ? 1 : 0; a.sink_values = sink ? sink_values : nullptr; a.scale = scale;
     const dim3 grid(n_seqs, Hkv * head_tiles, n_splits);
     int rc = BN_ERR_ARG;
     switch (hs / 32) {
@@ -474,6 +480,6 @@ extern "C" int bn_attn_general_decode(const void* q, int q_stride, void* out, in
     }
     if (rc != 0 || n_splits == 1) return rc;
     hipLaunchKernelGGL(attn_general_combine_kernel, dim3(n_seqs * H), dim3(BN_WAVE), 0, s, (bf16*)out, out_stride, part_o, part_ml,
-                       H, vd, n_splits, sink ? 1 : 0);
+                       H, vd, n_splits, sink ? 1 : 0, sink ? sink_values : nullptr);
     return bn_launch_status();
 }

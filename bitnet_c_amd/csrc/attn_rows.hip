@@ -45,7 +45,8 @@ struct AttnArgs {
                               // value pages are vd wide
     const float* dist_a;      // [H] or null: a bias that grows with the distance is taken off the score of query i and
     const float* dist_b;      // key j: dist_a[h] * ln(1 + dist_b[h] * (i - j))
-    int sink;                 // 1: the softmax has one more term of score 0 and no value (1 is added to its denominator)
+    int sink;                 // 1: the softmax has one more term without a value: exp(sink_values[head]) joins its denominator
+    const float* sink_values; // [H] float32, or null: the term's score is 0 for every head
 };
 
 // The fold of one run of keys into the sums of the runs before it: (M, L, O) <- (M, L, O) + (m, l, o) with both sides
@@ -58,11 +59,11 @@ __device__ __forceinline__ void fold_factors(float M, float m, float& m2, float&
 }
 __device__ __forceinline__ float fold_value(float O, float fa, float o, float fb) { return __fmaf_rn(O, fa, __fmul_rn(o, fb)); }
 
-// The sink of a softmax, as one more run of keys with maximum 0, sum 1 and no values, folded last with the operations of a
-// fold: every path (one workgroup, folded runs, merged splits) ends with the same step.
-__device__ __forceinline__ void fold_sink(float& M, float& L, float& fa) {
+// The sink of a softmax, as one more run of keys with maximum sv (the sink's score), sum 1 and no values, folded last with
+// the operations of a fold: every path (one workgroup, folded runs, merged splits) ends with the same step.
+__device__ __forceinline__ void fold_sink(float& M, float& L, float& fa, float sv) {
     float m2, fb;
-    fold_factors(M, 0.f, m2, fa, fb);                    // fa = 0 when the row saw no key
+    fold_factors(M, sv, m2, fa, fb);                     // fa = 0 when the row saw no key
     L = fold_value(L, fa, 1.f, fb);
     M = m2;
 }
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
             float o0 = folded ? tot[r][0] : acc[r][0], o1 = folded ? tot[r][1] : acc[r][1];
             if (a.sink) {
                 float m = folded ? Mt_s[r] : m_s[r], fa;
-                fold_sink(m, l, fa);
+                fold_sink(m, l, fa, a.sink_values ? a.sink_values[head] : 0.f);
                 o0 = __fmul_rn(o0, fa); o1 = __fmul_rn(o1, fa);
             }
             const float inv = l > 0.f ? 1.0f / l : 0.f;
@@ -406,14 +407,16 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_rows_kernel(AttnArgs a) {
 // out[row, d] = sum_s e^{m_s - m} o_s[d] / sum_s e^{m_s - m} l_s, splits in index order
 template <typename T>
 __global__ void attn_combine_kernel(T* __restrict__ out, int out_stride, const float* __restrict__ part_o,
-                                    const float* __restrict__ part_ml, int H, int hs, int n_splits, int sink) {
+                                    const float* __restrict__ part_ml, int H, int hs, int n_splits, int sink,
+                                    const float* __restrict__ sink_values) {
     const int row = blockIdx.x;               // token*H + head; hs: the width of a value head
     const int tok = row / H, head = row - tok * H;
     const float* ml = part_ml + (size_t)row * n_splits * 2;
-    float m = sink ? 0.f : -INFINITY;
+    const float sv = sink && sink_values ? sink_values[head] : 0.f;
+    float m = sink ? sv : -INFINITY;
     for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
     for (int d = threadIdx.x; d < hs; d += blockDim.x) {
-        float num = 0.f, den = sink ? expf(-m) : 0.f;
+        float num = 0.f, den = sink ? expf(sv - m) : 0.f;
         if (m != -INFINITY) {
             for (int s = 0; s < n_splits; ++s) {
                 const float w = expf(ml[2 * s] - m);          // 0 for an empty split
@@ -429,10 +432,12 @@ __global__ void attn_combine_kernel(T* __restrict__ out, int out_stride, const f
 // operations of fold_factors and fold_value, which is what a workgroup that walks all runs by itself does; runs without keys are passed over.
 template <typename T>
 __global__ void attn_fold_kernel(T* __restrict__ out, int out_stride, const float* __restrict__ part_o,
-                                 const float* __restrict__ part_ml, int H, int hs, int n_splits, int sink) {
+                                 const float* __restrict__ part_ml, int H, int hs, int n_splits, int sink,
+                                 const float* __restrict__ sink_values) {
     const int row = blockIdx.x;               // token*H + head; hs: the width of a value head
     const int tok = row / H, head = row - tok * H;
     const float* ml = part_ml + (size_t)row * n_splits * 2;
+    const float sv = sink && sink_values ? sink_values[head] : 0.f;
     for (int d = threadIdx.x; d < hs; d += blockDim.x) {
         float M = -INFINITY, L = 0.f, O = 0.f;
         for (int s = 0; s < n_splits; ++s) {
@@ -444,7 +449,7 @@ __global__ void attn_fold_kernel(T* __restrict__ out, int out_stride, const floa
             O = fold_value(O, fa, part_o[((size_t)row * n_splits + s) * hs + d], fb);
             M = m2;
         }
-        if (sink) { float fa; fold_sink(M, L, fa); O = __fmul_rn(O, fa); }
+        if (sink) { float fa; fold_sink(M, L, fa, sv); O = __fmul_rn(O, fa); }
         const float inv = L > 0.f ? 1.0f / L : 0.f;
         out[(size_t)tok * out_stride + (size_t)head * hs + d] = from_f32<T>(__fmul_rn(O, inv));
     }
@@ -503,7 +508,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
                             int n_tokens, int H, int Hkv, int hs, int RT, int GT, int window,
                             float scale, int n_splits, int chunk, float* part_o, float* part_ml,
                             int v_transposed, const int* max_len, int fold, int vd, const float* dist_a,
-                            const float* dist_b, int sink, hipStream_t s) {
+                            const float* dist_b, int sink, const float* sink_values, hipStream_t s) {
     if (vd == 0) vd = hs;
     if (vd < 2 || vd > BN_MAX_HEAD_DIM || vd % 2 || (dist_a == nullptr) != (dist_b == nullptr)) return BN_ERR_ARG;
     if (n_tiles <= 0 || n_tokens <= 0 || H <= 0 || Hkv <= 0 || H % Hkv) return BN_ERR_ARG;
@@ -526,7 +531,7 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     a.scale = scale;
     a.v_transposed = v_transposed;
     a.fold = fold;
-    a.vd = vd; a.dist_a = dist_a; a.dist_b = dist_b; a.sink = sink ? 1 : 0;
+    a.vd = vd; a.dist_a = dist_a; a.dist_b = dist_b; a.sink = sink ? 1 : 0; a.sink_values = sink ? sink_values : nullptr;
     a.KT = attn_key_tile(dtype, hs, vd);
     if (a.KT == 0) return BN_ERR_ARG;
     int rc;
@@ -537,17 +542,17 @@ extern "C" int bn_attn_rows(int dtype, const void* q, int q_stride, void* out, i
     if (fold > 0) {
         if (dtype == BN_DT_F32)
             hipLaunchKernelGGL(attn_fold_kernel<float>, dim3(n_tokens * H), dim3(64), 0, s, (float*)out, out_stride, part_o,
-                               part_ml, H, vd, n_splits, a.sink);
+                               part_ml, H, vd, n_splits, a.sink, a.sink_values);
         else
             hipLaunchKernelGGL(attn_fold_kernel<bf16>, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out, out_stride, part_o,
-                               part_ml, H, vd, n_splits, a.sink);
+                               part_ml, H, vd, n_splits, a.sink, a.sink_values);
         return bn_launch_status();
     }
     if (dtype == BN_DT_F32)
         hipLaunchKernelGGL(attn_combine_kernel<float>, dim3(n_tokens * H), dim3(64), 0, s, (float*)out,
-                           out_stride, part_o, part_ml, H, vd, n_splits, a.sink);
+                           out_stride, part_o, part_ml, H, vd, n_splits, a.sink, a.sink_values);
     else
         hipLaunchKernelGGL(attn_combine_kernel<bf16>, dim3(n_tokens * H), dim3(64), 0, s, (bf16*)out,
-                           out_stride, part_o, part_ml, H, vd, n_splits, a.sink);
+                           out_stride, part_o, part_ml, H, vd, n_splits, a.sink, a.sink_values);
     return bn_launch_status();
 }

@@ -24,7 +24,7 @@ ARCH = "gfx950"
 # -packed-fp32-ops off: hipcc otherwise forms packed float32 instructions by itself
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
-SOURCES = ("elementwise", "rope_kv", "qk_norm", "attn_rows", "attn_mfma", "attn_mfma_general", "state_mixers", "lightning", "latent", "moe", "gemm_tiled", "gemm_mfma", "skinny_gemm",
+SOURCES = ("elementwise", "rope_kv", "qk_norm", "attn_rows", "attn_mfma", "attn_mfma_general", "state_mixers", "lightning", "conv_scans", "hyper", "latent", "moe", "gemm_tiled", "gemm_mfma", "skinny_gemm",
            "splitk_gemm", "sampling")
 HEADERS = ("common.h", "attn_mfma.h")
 

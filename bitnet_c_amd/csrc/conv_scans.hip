@@ -1,0 +1,378 @@
+// Short causal convolutions over time and two recurrences with a float32 state per sequence.
+//
+//   bn_short_conv   y_t = sum_j w[:, j] u_(t - taps + 1 + j) (+ bias) on every channel of a projection, zeros before a
+//                   sequence's first token.  The last taps - 1 inputs of a sequence are part of its state: a step's
+//                   first tokens read them from there, and the step leaves its own last inputs behind.
+//   bn_lru_gates    the gates of a real-gated linear recurrent unit: the input in `blocks` equal parts, in part b
+//                   r = sigmoid(Wa[b] u_b + ba), i = sigmoid(Wi[b] u_b + bi); a = exp(c r) with c = -8 softplus(lam) per
+//                   channel; the unit's two operands a and sqrt(1 - a^2) i u leave as float32 rows
+//   bn_lru_scan     S <- a S + b per channel, the result times gelu_tanh of the other branch
+//   bn_gla_scan     gated linear attention: per head S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T q_t with a decay per key
+//                   channel and token, alpha = sigmoid(z)^(1 / tau)
+//
+// Everything that enters a recurrence is float32: gates, decays and their logarithms, exponentials, the state.  Every
+// chain is the same operations in the same order whatever else a step holds, so a sequence's values do not depend on
+// how its tokens were cut into steps or on the batch.
+#include "common.h"
+#include <math.h>
+
+#define BN_CONV_MAX_TAPS 16       // the Python side reads this line
+#define GLA_MAX_DIM 256           // key channels of a head (the Python side reads this line)
+#define GLA_COLS 16               // value columns of a wave
+#define GLA_SLICES 4              // parts of the key channels, 16 lanes each
+#define GLA_RUN 16                // tokens staged at once
+
+struct SeqRange { int seq, row0, n, pos0; };
+
+__device__ __forceinline__ SeqRange seq_range(const int* tiles, const int* seq_lens, int idx) {
+    SeqRange r;
+    if (tiles) {
+        const int* t = tiles + 4 * idx;
+        r.seq = t[0]; r.row0 = t[1]; r.n = t[2]; r.pos0 = t[3];
+    } else {
+        r.seq = idx; r.row0 = idx; r.pos0 = seq_lens[idx] - 1; r.n = r.pos0 >= 0 ? 1 : 0;
+    }
+    return r;
+}
+
+// ---- short convolution ----------------------------------------------------------------------------------------------
+struct ConvArgs {
+    const void* x;            // [T, ldx]; the channels start at column col
+    void* y;                  // [T, ldy]: the channels from column 0
+    const float* w;           // [C, taps]; the last column meets the current token
+    const float* bias;        // [C] or null
+    float* state;             // row of a slot: [taps - 1][C], the inputs before the step's first token, oldest first
+    const int* positions;     // [T]; < 0: a padding row
+    const int* seq_index;     // [T]
+    const int* slot_ids;      // [sequences]
+    const int* tiles;         // [n, 4] one tile a sequence (prompt form) or null
+    const int* seq_lens;      // decode form: row b is sequence b's one token
+    long long state_stride;
+    int ldx, ldy, col, T, C, taps;
+};
+
+// One thread a (row, channel).  The token j places back is the row j places up when that row is the same sequence's
+// token at that position; from the first j0 for which it is not, the state holds it: position pos0 - 1 - (j - j0) is
+// state entry taps - 2 - (j - j0).  Reads the state only.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void short_conv_rows_kernel(ConvArgs a) {
+    const int t = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= a.C) return;
+    TO* y = reinterpret_cast<TO*>(a.y) + (size_t)t * a.ldy + c;
+    const int pos = a.positions[t];
+    if (pos < 0) { *y = from_f32<TO>(0.f); return; }
+    const int seq = a.seq_index[t];
+    const TI* x = reinterpret_cast<const TI*>(a.x) + a.col + c;
+    const float* w = a.w + (size_t)c * a.taps;
+    const float* st = a.state + (size_t)a.slot_ids[seq] * a.state_stride + c;
+    float acc = a.bias ? a.bias[c] : 0.f;
+    int j0 = -1;
+    for (int j = 0; j < a.taps && j <= pos; ++j) {
+        if (j0 < 0 && !(t - j >= 0 && a.seq_index[t - j] == seq && a.positions[t - j] == pos - j)) j0 = j;
+        const float u = j0 < 0 ? to_f32(x[(size_t)(t - j) * a.ldx]) : st[(size_t)(a.taps - 2 - (j - j0)) * a.C];
+        acc = fmaf(w[a.taps - 1 - j], u, acc);
+    }
+    *y = from_f32<TO>(acc);
+}
+
+// One thread a (sequence, channel): the state after the step holds the inputs at the last taps - 1 positions, which are
+// rows of the step or, for a step shorter than that, entries of the old state further up (read before they are written).
+template <typename TI>
+__global__ __launch_bounds__(256) void short_conv_state_kernel(ConvArgs a) {
+    const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (sr.n <= 0 || sr.pos0 < 0 || c >= a.C) return;
+    const TI* x = reinterpret_cast<const TI*>(a.x) + a.col + c;
+    float* st = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + c;
+    const int keep = a.taps - 1;
+    for (int i = 0; i < keep; ++i) {
+        const int p = sr.pos0 + sr.n - keep + i;             // the position that entry i will hold
+        float v = 0.f;
+        if (p >= sr.pos0) v = to_f32(x[(size_t)(sr.row0 + (p - sr.pos0)) * a.ldx]);
+        else if (p >= 0) v = st[(size_t)(keep + (p - sr.pos0)) * a.C];
+        st[(size_t)i * a.C] = v;
+    }
+}
+
+// Decode form, both in one: one thread a (sequence, channel) reads the state and the new input, leaves the output and
+// the state moved on by one.
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void short_conv_decode_kernel(ConvArgs a) {
+    const int b = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= a.C) return;
+    TO* y = reinterpret_cast<TO*>(a.y) + (size_t)b * a.ldy + c;
+    const int pos = a.seq_lens[b] - 1;
+    if (pos < 0) { *y = from_f32<TO>(0.f); return; }
+    const float u0 = to_f32(reinterpret_cast<const TI*>(a.x)[(size_t)b * a.ldx + a.col + c]);
+    const float* w = a.w + (size_t)c * a.taps;
+    float* st = a.state + (size_t)a.slot_ids[b] * a.state_stride + c;
+    const int keep = a.taps - 1;
+    float acc = fmaf(w[keep], u0, a.bias ? a.bias[c] : 0.f);
+    for (int j = 1; j <= keep; ++j) {                       // the token j places back is state entry keep - j
+        const float u = j <= pos ? st[(size_t)(keep - j) * a.C] : 0.f;
+        acc = fmaf(w[keep - j], u, acc);
+    }
+    for (int i = 0; i + 1 < keep; ++i) st[(size_t)i * a.C] = (keep - 1 - i) <= pos ? st[(size_t)(i + 1) * a.C] : 0.f;
+    if (keep > 0) st[(size_t)(keep - 1) * a.C] = u0;
+    *y = from_f32<TO>(acc);
+}
+
+// in_dtype: x's type; out_dtype: y's.  n_seqs: tiles (prompt form) or sequences (decode form: tiles null, seq_lens given).
+extern "C" int bn_short_conv(int in_dtype, int out_dtype, const void* x, int ldx, int col, void* y, int ldy, const float* w,
+                             const float* bias, float* state, long long state_stride, const int* positions,
+                             const int* seq_index, const int* slot_ids, const int* tiles, const int* seq_lens, int n_seqs,
+                             int T, int C, int taps, hipStream_t s) {
+    if (T <= 0 || C <= 0 || taps < 1 || taps > BN_CONV_MAX_TAPS || n_seqs <= 0) return BN_ERR_ARG;
+    if (!x || !y || !w || !state || !positions || !seq_index || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
+    if (ldx < col + C || ldy < C || state_stride < (long long)(taps - 1) * C) return BN_ERR_ARG;
+    if (!tiles && n_seqs != T) return BN_ERR_ARG;
+    ConvArgs a;
+    a.x = x; a.y = y; a.w = w; a.bias = bias; a.state = state; a.positions = positions; a.seq_index = seq_index;
+    a.slot_ids = slot_ids; a.tiles = tiles; a.seq_lens = seq_lens; a.state_stride = state_stride; a.ldx = ldx; a.ldy = ldy;
+    a.col = col; a.T = T; a.C = C; a.taps = taps;
+    const int threads = C >= 256 ? 256 : 64;
+    const int cb = (C + threads - 1) / threads;
+    const bool fi = in_dtype == BN_DT_F32, fo = out_dtype == BN_DT_F32;
+    if ((!fi && in_dtype != BN_DT_BF16) || (!fo && out_dtype != BN_DT_BF16)) return BN_ERR_DTYPE;
+    if (!tiles) {
+        const dim3 grid(T, cb);
+        if (fi && fo) hipLaunchKernelGGL((short_conv_decode_kernel<float, float>), grid, dim3(threads), 0, s, a);
+        else if (fi) hipLaunchKernelGGL((short_conv_decode_kernel<float, bf16>), grid, dim3(threads), 0, s, a);
+        else if (fo) hipLaunchKernelGGL((short_conv_decode_kernel<bf16, float>), grid, dim3(threads), 0, s, a);
+        else hipLaunchKernelGGL((short_conv_decode_kernel<bf16, bf16>), grid, dim3(threads), 0, s, a);
+        return bn_launch_status();
+    }
+    const dim3 grid(T, cb);
+    if (fi && fo) hipLaunchKernelGGL((short_conv_rows_kernel<float, float>), grid, dim3(threads), 0, s, a);
+    else if (fi) hipLaunchKernelGGL((short_conv_rows_kernel<float, bf16>), grid, dim3(threads), 0, s, a);
+    else if (fo) hipLaunchKernelGGL((short_conv_rows_kernel<bf16, float>), grid, dim3(threads), 0, s, a);
+    else hipLaunchKernelGGL((short_conv_rows_kernel<bf16, bf16>), grid, dim3(threads), 0, s, a);
+    if (taps > 1) {
+        const dim3 sgrid(n_seqs, cb);
+        if (fi) hipLaunchKernelGGL(short_conv_state_kernel<float>, sgrid, dim3(threads), 0, s, a);
+        else hipLaunchKernelGGL(short_conv_state_kernel<bf16>, sgrid, dim3(threads), 0, s, a);
+    }
+    return bn_launch_status();
+}
+
+// ---- gates of the real-gated linear recurrent unit ----------------------------------------------------------------
+#define LRU_ROWS 8
+#define LRU_COLS 128
+
+// One workgroup a (eight rows, block of the input, 128 output channels of the block).  The rows' part of u is staged in
+// shared memory; a thread owns an output channel and walks the part's inputs in order with both matrices, which lie
+// [block][in][out] so that the threads of a wave read neighbouring words.
+__global__ __launch_bounds__(LRU_COLS) void lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ wa,
+                                                             const float* __restrict__ ba, const float* __restrict__ wi,
+                                                             const float* __restrict__ bi, const float* __restrict__ c_neg,
+                                                             float* __restrict__ a_out, float* __restrict__ b_out, int T,
+                                                             int W, int bw) {
+    extern __shared__ float us[];                        // [LRU_ROWS][bw]
+    const int t0 = blockIdx.x * LRU_ROWS, blk = blockIdx.y, o = blockIdx.z * LRU_COLS + threadIdx.x;
+    const int rows = min(LRU_ROWS, T - t0);
+    for (int idx = threadIdx.x; idx < LRU_ROWS * bw; idx += LRU_COLS) {
+        const int r = idx / bw, i = idx - r * bw;
+        us[idx] = r < rows ? u[(size_t)(t0 + r) * W + (size_t)blk * bw + i] : 0.f;
+    }
+    __syncthreads();
+    if (o >= bw) return;
+    float acc_a[LRU_ROWS], acc_i[LRU_ROWS];
+#pragma unroll
+    for (int r = 0; r < LRU_ROWS; ++r) { acc_a[r] = 0.f; acc_i[r] = 0.f; }
+    const float* pa = wa + (size_t)blk * bw * bw + o;
+    const float* pi = wi + (size_t)blk * bw * bw + o;
+#pragma unroll 4
+    for (int i = 0; i < bw; ++i) {
+        const float va = pa[(size_t)i * bw], vi = pi[(size_t)i * bw];
+#pragma unroll
+        for (int r = 0; r < LRU_ROWS; ++r) {
+            const float x = us[r * bw + i];
+            acc_a[r] = fmaf(va, x, acc_a[r]);
+            acc_i[r] = fmaf(vi, x, acc_i[r]);
+        }
+    }
+    const int ch = blk * bw + o;
+    const float biasa = ba[ch], biasi = bi[ch], cn = c_neg[ch];
+#pragma unroll
+    for (int r = 0; r < LRU_ROWS; ++r) {
+        if (r >= rows) break;
+        const float rg = 1.0f / (1.0f + expf(-(acc_a[r] + biasa)));
+        const float ig = 1.0f / (1.0f + expf(-(acc_i[r] + biasi)));
+        const float la = cn * rg;                                  // log a <= 0
+        const float m = sqrtf(fmaxf(-expm1f(2.0f * la), 0.f));      // sqrt(1 - a^2) without the cancellation near a = 1
+        a_out[(size_t)(t0 + r) * W + ch] = expf(la);
+        b_out[(size_t)(t0 + r) * W + ch] = m * ig * us[r * bw + o];
+    }
+}
+
+extern "C" int bn_lru_gates(const float* u, const float* wa, const float* ba, const float* wi, const float* bi,
+                            const float* c_neg, float* a_out, float* b_out, int T, int W, int blocks, hipStream_t s) {
+    if (T <= 0 || W <= 0 || blocks <= 0 || W % blocks || !u || !wa || !ba || !wi || !bi || !c_neg || !a_out || !b_out) return BN_ERR_ARG;
+    const int bw = W / blocks;
+    const size_t shm = (size_t)LRU_ROWS * bw * sizeof(float);
+    const int row_tiles = (T + LRU_ROWS - 1) / LRU_ROWS;
+    if (shm > 64 * 1024 || blocks > 65535 || (bw + LRU_COLS - 1) / LRU_COLS > 65535) return BN_ERR_ARG;
+    const dim3 grid(row_tiles, blocks, (bw + LRU_COLS - 1) / LRU_COLS);
+    hipLaunchKernelGGL(lru_gates_kernel, grid, dim3(LRU_COLS), shm, s, u, wa, ba, wi, bi, c_neg, a_out, b_out, T, W, bw);
+    return bn_launch_status();
+}
+
+// ---- S <- a S + b, times the other branch ---------------------------------------------------------------------------
+#define LRU_AHEAD 8
+
+// One thread a (sequence, channel) walks the sequence's tokens; the loads of the next LRU_AHEAD tokens are in flight
+// while the chain advances.
+template <typename T>
+__global__ __launch_bounds__(64) void lru_scan_kernel(const float* __restrict__ av, const float* __restrict__ bv,
+                                                      const T* __restrict__ ypre, int ldy, T* __restrict__ out,
+                                                      float* __restrict__ state, long long state_stride,
+                                                      const int* __restrict__ tiles, const int* __restrict__ seq_lens,
+                                                      const int* __restrict__ slot_ids, int W) {
+    const SeqRange sr = seq_range(tiles, seq_lens, blockIdx.x);
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (sr.n <= 0 || sr.pos0 < 0 || c >= W) return;
+    float* sp = state + (size_t)slot_ids[sr.seq] * state_stride + c;
+    float S = sr.pos0 > 0 ? *sp : 0.f;
+    const float* ap = av + (size_t)sr.row0 * W + c;
+    const float* bp = bv + (size_t)sr.row0 * W + c;
+    const T* yp = ypre + (size_t)sr.row0 * ldy + c;
+    T* op = out + (size_t)sr.row0 * W + c;
+    for (int t0 = 0; t0 < sr.n; t0 += LRU_AHEAD) {
+        float a[LRU_AHEAD], b[LRU_AHEAD], y[LRU_AHEAD];
+#pragma unroll
+        for (int i = 0; i < LRU_AHEAD; ++i) {
+            const int t = min(t0 + i, sr.n - 1);
+            a[i] = ap[(size_t)t * W]; b[i] = bp[(size_t)t * W]; y[i] = to_f32(yp[(size_t)t * ldy]);
+        }
+#pragma unroll
+        for (int i = 0; i < LRU_AHEAD; ++i) {
+            if (t0 + i >= sr.n) break;
+            S = fmaf(a[i], S, b[i]);
+            op[(size_t)(t0 + i) * W] = from_f32<T>(S * bn_gate_act(y[i], BN_ACT_GELU_TANH));
+        }
+    }
+    *sp = S;
+}
+
+extern "C" int bn_lru_scan(int dtype, const float* av, const float* bv, const void* ypre, int ldy, void* out, float* state,
+                           long long state_stride, const int* tiles, int n_seqs, const int* seq_lens, const int* slot_ids,
+                           int W, hipStream_t s) {
+    if (n_seqs <= 0 || W <= 0 || !av || !bv || !ypre || !out || !state || !slot_ids || (!tiles && !seq_lens) || ldy < W) return BN_ERR_ARG;
+    if (state_stride < W) return BN_ERR_ARG;
+    const dim3 grid(n_seqs, (W + 63) / 64);
+    if (dtype == BN_DT_F32)
+        hipLaunchKernelGGL(lru_scan_kernel<float>, grid, dim3(64), 0, s, av, bv, (const float*)ypre, ldy, (float*)out, state,
+                           state_stride, tiles, seq_lens, slot_ids, W);
+    else if (dtype == BN_DT_BF16)
+        hipLaunchKernelGGL(lru_scan_kernel<bf16>, grid, dim3(64), 0, s, av, bv, (const bf16*)ypre, ldy, (bf16*)out, state,
+                           state_stride, tiles, seq_lens, slot_ids, W);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- gated linear attention -----------------------------------------------------------------------------------------
+struct GlaArgs {
+    const void* x;            // [T, ld]: q at q_col, k at k_col (head h at h * dk), v at v_col (head h at h * dv)
+    const float* z;           // [T, H dk]: the decay's logits, bias included
+    float* o;                 // [T, H dv] float32
+    float* state;             // row of a slot: [H][dk][dv]
+    const int* tiles;
+    const int* seq_lens;
+    const int* slot_ids;
+    long long state_stride;
+    int ld, q_col, k_col, v_col, H, dk, dv;
+    float q_scale, inv_tau;
+};
+
+// A wave owns (sequence, head, 16 value columns).  Lane = (slice s of the key channels, column c): it keeps rows
+// s, s + 4, s + 8, ... of its column of S in registers.  Tokens come in runs of 16: the wave stages q (scaled), k and
+// alpha of the run as float32 in shared memory (alpha = exp(logsigmoid(z) / tau)), then walks the run; the four slices'
+// parts of o meet through two lane exchanges in a fixed order.
+template <typename T, int RPL>
+__global__ __launch_bounds__(BN_WAVE) void gla_scan_kernel(GlaArgs a) {
+    constexpr int DKP = GLA_SLICES * RPL;                 // staged key channels (those past dk are zeros)
+    __shared__ float q_s[GLA_RUN][DKP], k_s[GLA_RUN][DKP], a_s[GLA_RUN][DKP], v_s[GLA_RUN][GLA_COLS];
+    const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
+    if (sr.n <= 0 || sr.pos0 < 0) return;
+    const int head = blockIdx.y, col0 = blockIdx.z * GLA_COLS;
+    const int lane = threadIdx.x, sl = lane >> 4, c = lane & 15;
+    const bool has = col0 + c < a.dv;
+    const T* x = reinterpret_cast<const T*>(a.x);
+    float* sp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * a.dk * a.dv + col0 + c;
+    float S[RPL];
+#pragma unroll
+    for (int r = 0; r < RPL; ++r) {
+        const int i = sl + GLA_SLICES * r;
+        S[r] = (sr.pos0 > 0 && has && i < a.dk) ? sp[(size_t)i * a.dv] : 0.f;
+    }
+    for (int t0 = 0; t0 < sr.n; t0 += GLA_RUN) {
+        const int run = min(GLA_RUN, sr.n - t0);
+        __syncthreads();
+        for (int idx = lane; idx < GLA_RUN * DKP; idx += BN_WAVE) {
+            const int tt = idx / DKP, i = idx - tt * DKP;
+            float qv = 0.f, kv = 0.f, al = 0.f;
+            if (tt < run && i < a.dk) {
+                const size_t row = (size_t)(sr.row0 + t0 + tt);
+                qv = to_f32(x[row * a.ld + a.q_col + head * a.dk + i]) * a.q_scale;
+                kv = to_f32(x[row * a.ld + a.k_col + head * a.dk + i]);
+                const float zz = a.z[row * (size_t)(a.H * a.dk) + (size_t)head * a.dk + i];
+                al = expf((fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * a.inv_tau);
+            }
+            q_s[tt][i] = qv; k_s[tt][i] = kv; a_s[tt][i] = al;
+        }
+        for (int idx = lane; idx < GLA_RUN * GLA_COLS; idx += BN_WAVE) {
+            const int tt = idx / GLA_COLS, cc = idx - tt * GLA_COLS;
+            v_s[tt][cc] = (tt < run && col0 + cc < a.dv)
+                              ? to_f32(x[(size_t)(sr.row0 + t0 + tt) * a.ld + a.v_col + head * a.dv + col0 + cc]) : 0.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < run; ++tt) {
+            const float vj = v_s[tt][c];
+            float o = 0.f;
+#pragma unroll
+            for (int r = 0; r < RPL; ++r) {
+                const int i = sl + GLA_SLICES * r;
+                S[r] = fmaf(a_s[tt][i], S[r], k_s[tt][i] * vj);
+                o = fmaf(S[r], q_s[tt][i], o);
+            }
+            o += __shfl_xor(o, 16, BN_WAVE);
+            o += __shfl_xor(o, 32, BN_WAVE);
+            if (sl == 0 && has) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col0 + c] = o;
+        }
+    }
+    if (has) {
+#pragma unroll
+        for (int r = 0; r < RPL; ++r) {
+            const int i = sl + GLA_SLICES * r;
+            if (i < a.dk) sp[(size_t)i * a.dv] = S[r];
+        }
+    }
+}
+
+extern "C" int bn_gla_supports(int dk, int dv) { return (dk >= 1 && dk <= GLA_MAX_DIM && dv >= 1) ? 1 : 0; }
+
+template <typename T>
+static int gla_launch(const GlaArgs& a, dim3 grid, hipStream_t s) {
+    const int rpl = (a.dk + GLA_SLICES - 1) / GLA_SLICES;
+    if (rpl <= 8) hipLaunchKernelGGL((gla_scan_kernel<T, 8>), grid, dim3(BN_WAVE), 0, s, a);
+    else if (rpl <= 16) hipLaunchKernelGGL((gla_scan_kernel<T, 16>), grid, dim3(BN_WAVE), 0, s, a);
+    else if (rpl <= 32) hipLaunchKernelGGL((gla_scan_kernel<T, 32>), grid, dim3(BN_WAVE), 0, s, a);
+    else hipLaunchKernelGGL((gla_scan_kernel<T, 64>), grid, dim3(BN_WAVE), 0, s, a);
+    return bn_launch_status();
+}
+
+extern "C" int bn_gla_scan(int dtype, const void* x, int ld, int q_col, int k_col, int v_col, const float* z, float* o,
+                           float* state, long long state_stride, const int* tiles, int n_seqs, const int* seq_lens,
+                           const int* slot_ids, int H, int dk, int dv, float q_scale, float inv_tau, hipStream_t s) {
+    if (n_seqs <= 0 || H <= 0 || !bn_gla_supports(dk, dv) || !x || !z || !o || !state || !slot_ids || (!tiles && !seq_lens)) return BN_ERR_ARG;
+    if (ld < q_col + H * dk || ld < k_col + H * dk || ld < v_col + H * dv || state_stride < (long long)H * dk * dv) return BN_ERR_ARG;
+    if (H > 65535 || (dv + GLA_COLS - 1) / GLA_COLS > 65535) return BN_ERR_ARG;
+    GlaArgs a;
+    a.x = x; a.z = z; a.o = o; a.state = state; a.tiles = tiles; a.seq_lens = seq_lens; a.slot_ids = slot_ids;
+    a.state_stride = state_stride; a.ld = ld; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col; a.H = H; a.dk = dk; a.dv = dv;
+    a.q_scale = q_scale; a.inv_tau = inv_tau;
+    const dim3 grid(n_seqs, H, (dv + GLA_COLS - 1) / GLA_COLS);
+    if (dtype == BN_DT_F32) return gla_launch<float>(a, grid, s);
+    if (dtype == BN_DT_BF16) return gla_launch<bf16>(a, grid, s);
+    return BN_ERR_DTYPE;
+}

@@ -12,15 +12,16 @@
 #include <math.h>
 
 struct LatentStoreArgs {
-    const void* x;            // [T, ld]; the latent's columns start at column `col`
+    const void* x;            // [T, ld]; the latent's columns start at column `col`, the rotated key part follows them
     const int* positions;     // [T]; < 0: a padding row, nothing is written
     const int* seq_index;     // [T] row of the block table
     const int* block_table;   // [n_seqs, bt_stride]
-    void* k_pages;            // [pages, 1, BN_PAGE, rank]
+    void* k_pages;            // [pages, 1, BN_PAGE, rank + rot]: the latent, then the rotated part
     void* v_pages;            // [pages, 1, rank, BN_PAGE]
     const float* w;           // [rank]
-    int ld, col, rank, bt_stride;
-    float eps;
+    const float* inv_freq;    // [rot / 2] or null (rot 0)
+    int ld, col, rank, bt_stride, rot;
+    float eps, rot_mult;      // rot_mult multiplies every cosine and sine
 };
 
 template <typename T>
@@ -35,23 +36,34 @@ __global__ __launch_bounds__(256) void latent_store_kernel(LatentStoreArgs a) {
     ss = block_sum(ss, scratch);
     const float f = 1.0f / sqrtf(ss / (float)a.rank + a.eps);
     const int page = a.block_table[(size_t)a.seq_index[t] * a.bt_stride + pos / BN_PAGE], slot = pos % BN_PAGE;
-    T* kd = reinterpret_cast<T*>(a.k_pages) + ((size_t)page * BN_PAGE + slot) * a.rank;
+    T* kd = reinterpret_cast<T*>(a.k_pages) + ((size_t)page * BN_PAGE + slot) * (a.rank + a.rot);
     T* vd = reinterpret_cast<T*>(a.v_pages) + (size_t)page * a.rank * BN_PAGE + slot;
     for (int d = threadIdx.x; d < a.rank; d += blockDim.x) {
         const T c = from_f32<T>(to_f32(x[d]) * f * a.w[d]);
         kd[d] = c;
         vd[(size_t)d * BN_PAGE] = c;
     }
+    // the key part that all heads share: not normed, dimension i turned with dimension i + rot / 2 by pos * f_i
+    const int half = a.rot / 2;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+        float sn, cs;
+        sincosf((float)pos * a.inv_freq[i], &sn, &cs);
+        sn *= a.rot_mult; cs *= a.rot_mult;
+        const float u = to_f32(x[a.rank + i]), v = to_f32(x[a.rank + half + i]);
+        kd[a.rank + i] = from_f32<T>(u * cs - v * sn);
+        kd[a.rank + half + i] = from_f32<T>(v * cs + u * sn);
+    }
 }
 
 extern "C" int bn_latent_store(int dtype, const void* x, int ld, int col, const int* positions, const int* seq_index,
                                const int* block_table, int bt_stride, void* k_pages, void* v_pages, const float* w, int n_tokens,
-                               int rank, float eps, hipStream_t s) {
-    if (n_tokens <= 0 || rank <= 0 || col < 0 || ld < col + rank) return BN_ERR_ARG;
+                               int rank, float eps, int rot, const float* inv_freq, float rot_mult, hipStream_t s) {
+    if (n_tokens <= 0 || rank <= 0 || col < 0 || rot < 0 || rot % 2 || ld < col + rank + rot || (rot > 0 && !inv_freq)) return BN_ERR_ARG;
     if (!x || !positions || !seq_index || !block_table || !k_pages || !v_pages || !w) return BN_ERR_ARG;
     LatentStoreArgs a;
     a.x = x; a.positions = positions; a.seq_index = seq_index; a.block_table = block_table; a.k_pages = k_pages;
     a.v_pages = v_pages; a.w = w; a.ld = ld; a.col = col; a.rank = rank; a.bt_stride = bt_stride; a.eps = eps;
+    a.rot = rot; a.inv_freq = inv_freq; a.rot_mult = rot_mult;
     const dim3 grid(n_tokens), block(rank > 128 ? 256 : 64);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(latent_store_kernel<float>, grid, block, 0, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(latent_store_kernel<bf16>, grid, block, 0, s, a);
@@ -68,8 +80,8 @@ struct HeadLinearArgs {
     const void* x;            // [T, ldx]: head h at h * I
     const void* w;            // [H, I, O]
     void* y;                  // [T, ldy]: head h at h * O
-    const void* gate;         // [T, ldg]: head h at h * O; null: none
-    int ldx, ldy, ldg, T, H, I, O;
+    const void* gate;         // [T, ldg]: the gate of output column n is entry n / gate_group (1: one a column; O: one a head); null: none
+    int ldx, ldy, ldg, T, H, I, O, gate_group;
 };
 
 // The rows of x are staged in shared memory as float32 and read by every lane of a wave at the same address; a lane owns
@@ -113,7 +125,7 @@ __global__ __launch_bounds__(HL_COLS * HL_SLICES) void head_linear_kernel(HeadLi
         float v = 0.f;
 #pragma unroll
         for (int k = 0; k < HL_SLICES; ++k) v += red[(k * HL_ROWS + r) * HL_COLS + c];
-        if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + (size_t)h * a.O + o])));
+        if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + ((size_t)h * a.O + o) / a.gate_group])));
         y[(size_t)(t0 + r) * a.ldy + (size_t)h * a.O + o] = from_f32<T>(v);
     }
 }
@@ -187,7 +199,7 @@ __global__ __launch_bounds__(HLW_THREADS) void head_linear_wide_kernel(HeadLinea
         const int r = idx / a.O, o = idx - r * a.O;
         float v = 0.f;
         for (int k = 0; k < groups; ++k) v += red[((size_t)k * HLW_ROWS + r) * a.O + o];
-        if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + (size_t)h * a.O + o])));
+        if (g) v *= 1.0f / (1.0f + expf(-to_f32(g[(size_t)(t0 + r) * a.ldg + ((size_t)h * a.O + o) / a.gate_group])));
         y[(size_t)(t0 + r) * a.ldy + (size_t)h * a.O + o] = from_f32<T>(v);
     }
 }
@@ -201,13 +213,14 @@ static bool hlw_takes(const void* w, int I, int O) {
 }
 
 extern "C" int bn_head_linear(int dtype, const void* x, int ldx, const void* w, void* y, int ldy, const void* gate, int ldg,
-                              int n_rows, int H, int I, int O, hipStream_t s) {
+                              int gate_group, int n_rows, int H, int I, int O, hipStream_t s) {
     if (n_rows <= 0 || H <= 0 || I <= 0 || O <= 0 || !x || !w || !y) return BN_ERR_ARG;
-    if (ldx < H * I || ldy < H * O || (gate && ldg < H * O) || (size_t)HL_ROWS * (I + HL_SLICES * HL_COLS) * sizeof(float) > 64 * 1024 || H > 65535) return BN_ERR_ARG;
+    if (gate && (gate_group < 1 || (H * O) % gate_group)) return BN_ERR_ARG;
+    if (ldx < H * I || ldy < H * O || (gate && ldg < H * O / gate_group) || (size_t)HL_ROWS * (I + HL_SLICES * HL_COLS) * sizeof(float) > 64 * 1024 || H > 65535) return BN_ERR_ARG;
     const int row_tiles = (n_rows + HL_ROWS - 1) / HL_ROWS;
     if (row_tiles > 65535) return BN_ERR_ARG;
     HeadLinearArgs a;
-    a.x = x; a.w = w; a.y = y; a.gate = gate; a.ldx = ldx; a.ldy = ldy; a.ldg = ldg; a.T = n_rows; a.H = H; a.I = I; a.O = O;
+    a.x = x; a.w = w; a.y = y; a.gate = gate; a.ldx = ldx; a.ldy = ldy; a.ldg = ldg; a.T = n_rows; a.H = H; a.I = I; a.O = O; a.gate_group = gate ? gate_group : 1;
     if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
     const bool wide = dtype == BN_DT_F32 ? hlw_takes<float>(w, I, O) : hlw_takes<bf16>(w, I, O);
     if (wide && (n_rows + HLW_ROWS - 1) / HLW_ROWS <= 65535) {
@@ -228,21 +241,58 @@ extern "C" int bn_head_linear(int dtype, const void* x, int ldx, const void* w, 
 
 // ---- y *= sigmoid(gate) ---------------------------------------------------------------------------------------------
 template <typename T>
-__global__ void sigmoid_gate_kernel(T* __restrict__ y, int ldy, const T* __restrict__ g, int ldg, int n_rows, int n_cols) {
+__global__ void sigmoid_gate_kernel(T* __restrict__ y, int ldy, const T* __restrict__ g, int ldg, int n_rows, int n_cols, int group) {
     const size_t n = (size_t)n_rows * n_cols;
     for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
         const size_t r = idx / n_cols, c = idx - r * n_cols;
-        const float v = to_f32(y[r * ldy + c]) / (1.0f + expf(-to_f32(g[r * ldg + c])));
+        const float v = to_f32(y[r * ldy + c]) / (1.0f + expf(-to_f32(g[r * ldg + c / group])));
         y[r * ldy + c] = from_f32<T>(v);
     }
 }
 
-extern "C" int bn_sigmoid_gate(int dtype, void* y, int ldy, const void* gate, int ldg, int n_rows, int n_cols, hipStream_t s) {
-    if (n_rows <= 0 || n_cols <= 0 || ldy < n_cols || ldg < n_cols || !y || !gate) return BN_ERR_ARG;
+extern "C" int bn_sigmoid_gate(int dtype, void* y, int ldy, const void* gate, int ldg, int group, int n_rows, int n_cols, hipStream_t s) {
+    if (n_rows <= 0 || n_cols <= 0 || group < 1 || n_cols % group || ldy < n_cols || ldg < n_cols / group || !y || !gate) return BN_ERR_ARG;
     const size_t n = (size_t)n_rows * n_cols;
     const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
-    if (dtype == BN_DT_F32) hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)y, ldy, (const float*)gate, ldg, n_rows, n_cols);
-    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(sigmoid_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)y, ldy, (const bf16*)gate, ldg, n_rows, n_cols);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(sigmoid_gate_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)y, ldy, (const float*)gate, ldg, n_rows, n_cols, group);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(sigmoid_gate_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)y, ldy, (const bf16*)gate, ldg, n_rows, n_cols, group);
+    else return BN_ERR_DTYPE;
+    return bn_launch_status();
+}
+
+// ---- a rotation of part of every head, in place ------------------------------------------------------------------------
+// x[t, h * head_stride + off + i] is turned with x[t, h * head_stride + off + i + rot / 2] by the angle pos_t * f_i; both
+// cosine and sine times `mult`.  Rows with position < 0 are left alone.  Angles, cosines and sines in float32.
+template <typename T>
+__global__ void rope_heads_kernel(T* __restrict__ x, int ld, const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  int n_rows, int H, int head_stride, int off, int rot, float mult) {
+    const int half = rot / 2;
+    const size_t n = (size_t)n_rows * H * half;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+        const int i = (int)(idx % half);
+        const size_t th = idx / half;
+        const int h = (int)(th % H);
+        const size_t t = th / H;
+        const int pos = positions[t];
+        if (pos < 0) continue;
+        float sn, cs;
+        sincosf((float)pos * inv_freq[i], &sn, &cs);
+        sn *= mult; cs *= mult;
+        T* p = x + t * ld + (size_t)h * head_stride + off;
+        const float u = to_f32(p[i]), v = to_f32(p[half + i]);
+        p[i] = from_f32<T>(u * cs - v * sn);
+        p[half + i] = from_f32<T>(v * cs + u * sn);
+    }
+}
+
+extern "C" int bn_rope_heads(int dtype, void* x, int ld, const int* positions, const float* inv_freq, int n_rows, int H,
+                             int head_stride, int off, int rot, float mult, hipStream_t s) {
+    if (n_rows <= 0 || H <= 0 || rot <= 0 || rot % 2 || off < 0 || head_stride < off + rot || ld < (H - 1) * head_stride + off + rot
+        || !x || !positions || !inv_freq) return BN_ERR_ARG;
+    const size_t n = (size_t)n_rows * H * (rot / 2);
+    const int blocks = (int)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+    if (dtype == BN_DT_F32) hipLaunchKernelGGL(rope_heads_kernel<float>, dim3(blocks), dim3(256), 0, s, (float*)x, ld, positions, inv_freq, n_rows, H, head_stride, off, rot, mult);
+    else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(rope_heads_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (bf16*)x, ld, positions, inv_freq, n_rows, H, head_stride, off, rot, mult);
     else return BN_ERR_DTYPE;
     return bn_launch_status();
 }

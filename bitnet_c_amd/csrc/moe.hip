@@ -2,7 +2,7 @@
 // W_down[e] glu(W_gate[e] x, W_up[e] x)  with the clamped unit  glu(g, u) = g' sigmoid(slope g') (u' + shift),
 // g' = min(g, limit), u' = clamp(u, -limit, limit)  (gate and up rows stacked, [E, 2 F, D]).
 //
-//   bn_moe_route     router logits z = W_r h in float32 (one workgroup a token), scores sigmoid(z) or softmax(z), the top_k
+//   bn_moe_route     router logits z = W_r h (+ a bias per expert) in float32 (one workgroup a token), scores sigmoid(z) or softmax(z), the top_k
 //                    largest (ties: the lower index; with a choice bias the largest score + bias, the weights staying the
 //                    plain scores), optionally divided by their sum (+ floor), times a constant -> expert ids and weights
 //                    [T, top_k]; optionally also sigmoid(w_g . h) per token, the gate of a shared expert
@@ -30,6 +30,7 @@ struct RouteArgs {
     float* wts;               // [T, K]
     int ld, D, E, K, scoring, renorm;
     const float* bias;        // [E] added to the scores for the choice alone; null: the choice goes by the scores
+    const float* zbias;       // [E] added to the logits themselves (a router with a bias); null: none
     const float* gate_w;      // [D]: gate_out[t] = sigmoid(gate_w . h); null: none
     float* gate_out;          // [T]
     float floor, scale;       // weights = score / (sum of the chosen + floor) (when renorm) * scale
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
         }
         s = wave_sum(s);
         if (lane == 0) {
-            if (e < a.E) zs[e] = s;
+            if (e < a.E) zs[e] = a.zbias ? s + a.zbias[e] : s;
             else a.gate_out[t] = 1.0f / (1.0f + expf(-s));
         }
     }
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(RouteArgs 
 
 extern "C" int bn_moe_route(int dtype, const void* h, int ld, const float* wr, int* ids, float* wts, int n_tokens, int D, int E,
                             int K, int scoring, int renorm, const float* bias, float floor, float scale, const float* gate_w,
-                            float* gate_out, hipStream_t s) {
+                            float* gate_out, const float* zbias, hipStream_t s) {
     if ((gate_w == nullptr) != (gate_out == nullptr) || ((uintptr_t)gate_w & 15) || !(floor >= 0.f)) return BN_ERR_ARG;
     if (n_tokens <= 0 || D <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || K <= 0 || K > E || ld < D || !h || !wr || !ids || !wts)
         return BN_ERR_ARG;
@@ -142,7 +143,7 @@ extern "C" int bn_moe_route(int dtype, const void* h, int ld, const float* wr, i
     if ((size_t)(D + 4 + E) * sizeof(float) > 64 * 1024 || ((uintptr_t)wr & 15)) return BN_ERR_ARG;
     RouteArgs a;
     a.h = h; a.wr = wr; a.ids = ids; a.wts = wts; a.ld = ld; a.D = D; a.E = E; a.K = K; a.scoring = scoring; a.renorm = renorm ? 1 : 0;
-    a.bias = bias; a.gate_w = gate_w; a.gate_out = gate_out; a.floor = floor; a.scale = scale;
+    a.bias = bias; a.zbias = zbias; a.gate_w = gate_w; a.gate_out = gate_out; a.floor = floor; a.scale = scale;
     const size_t shm = (size_t)(((D + 3) & ~3) + E) * sizeof(float);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(moe_route_kernel<float>, dim3(n_tokens), dim3(MOE_ROUTE_THREADS), shm, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(moe_route_kernel<bf16>, dim3(n_tokens), dim3(MOE_ROUTE_THREADS), shm, s, a);

@@ -11,6 +11,7 @@ import torch
 
 from .. import ops
 from ..parts import BLOCKS, NORMS, CacheNeed, ResidualStream
+from ..parts.hyper import HyperStream
 from ..parts.linear import Linear, upload
 from .plan import ModelPlan
 
@@ -177,7 +178,10 @@ class DecoderModel:
                                           self.plan.embedding_multiplier)
         else:
             x = ops.embed_gather(self.embedding, ctx.tokens, self.plan.embedding_multiplier)    # src/model_embed.c:6-28
-        stream = ResidualStream(x)
+        if self.plan.residual_streams > 0:
+            stream = HyperStream(x, self.plan.residual_streams)
+        else:
+            stream = ResidualStream(x)
         for i, e in enumerate(self.plan.schedule):
             ctx.entry = i
             self.blocks[e.layer].forward(stream, ctx, views[i])

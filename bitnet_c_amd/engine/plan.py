@@ -50,6 +50,9 @@ class ModelPlan:
     # embedding row, entry 2i = sin(p base^(-2i/hidden)), entry 2i + 1 = cos of the same angle.
     position_sinusoid_base: float = 0.0
     logit_scale: float = 1.0             # the logits times this (before a bias or a soft-cap)
+    # > 0: the residual is that many float32 streams (parts/hyper.py: HyperStream, read and written by "hyper" blocks) that
+    # all start as the embedding's rows and are summed in front of the final norm; 0: the one stream of the other blocks.
+    residual_streams: int = 0
 
     def validate(self) -> None:
         if not self.embedding_multiplier > 0 or self.logit_softcap < 0:
@@ -57,6 +60,8 @@ class ModelPlan:
         if self.position_sinusoid_base < 0 or self.position_sinusoid_base == 1 or not self.logit_scale > 0:
             raise ValueError("the base of a sinusoidal position vector is 0 (none) or a positive number other than 1, "
                              "and the logits' multiplier is positive")
+        if self.residual_streams < 0:
+            raise ValueError("the number of residual streams is 0 (the plain residual) or positive")
         for i, e in enumerate(self.schedule):
             if not 0 <= e.layer < len(self.layers):
                 raise ValueError(f"schedule entry {i} names layer {e.layer}; there are {len(self.layers)}")

@@ -59,14 +59,15 @@ _SIGNATURES = {
     },
     "latent": {
         "bn_latent_store": [c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                            c_int, c_int, c_float, c_void_p],
-        "bn_head_linear": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                            c_int, c_int, c_float, c_int, c_void_p, c_float, c_void_p],
+        "bn_head_linear": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                            c_void_p],
-        "bn_sigmoid_gate": [c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+        "bn_sigmoid_gate": [c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_rope_heads": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p],
     },
     "moe": {
         "bn_moe_route": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
-                         c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p],
+                         c_void_p, c_float, c_float, c_void_p, c_void_p, c_void_p, c_void_p],
         "bn_moe_experts": [c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                            c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, c_void_p],
         "bn_gated_unit": [c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_float, c_float, c_float, c_void_p],
@@ -77,10 +78,26 @@ _SIGNATURES = {
     "attn_mfma_general": {
         "bn_attn_general_supports": [c_int, c_int],
         "bn_attn_general_prompt": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_void_p],
+                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p],
         "bn_attn_general_decode": [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p,
+                                   c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p,
                                    c_void_p, c_void_p, c_void_p],
+    },
+    "hyper": {
+        "bn_hc_step": [c_int, c_int, c_void_p, c_longlong, c_void_p, c_longlong, c_void_p, c_int, c_longlong, c_void_p, c_void_p,
+                       c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_dyt_norm": [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    },
+    "conv_scans": {
+        "bn_short_conv": [c_int, c_int, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_longlong,
+                          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "bn_lru_gates": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                         c_void_p],
+        "bn_lru_scan": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p,
+                        c_void_p, c_int, c_void_p],
+        "bn_gla_supports": [c_int, c_int],
+        "bn_gla_scan": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int,
+                        c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p],
     },
     "lightning": {
         "bn_lightning_supports": [c_int, c_int],
@@ -114,7 +131,7 @@ _SIGNATURES = {
         "bn_attn_rows_key_tile": [c_int, c_int],
         "bn_attn_rows": [c_int, c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                          c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                         c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p],
+                         c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p],
     },
     "attn_mfma": {
         "bn_attn_mfma_supports": [c_int],
@@ -1198,6 +1215,19 @@ def can_fuse_decode(dtype, H: int, Hkv: int, hs: int) -> bool:
     return mfma_attention(dtype, hs) and H // Hkv <= 16
 
 
+def _sink_args(sink, H: int, what: str):
+    """(flag, address) of a softmax's sink as the kernels take it: False or None, no sink; True, one more term of score
+    0; a float32 tensor [H], one more term of that score per head."""
+    if sink is None or sink is False:
+        return 0, None
+    if sink is True:
+        return 1, None
+    _dev(sink, "sink", torch.float32, 1)
+    if sink.numel() != H or not sink.is_contiguous():
+        raise KernelError(f"{what}: a sink with scores holds one float32 per head ({H}), got {tuple(sink.shape)}")
+    return 1, sink.data_ptr()
+
+
 def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               block_table: torch.Tensor, H: int, Hkv: int, hs: int, scale: float, *, window: int = 0,
               tiles=None, qt: int = 0, seq_lens=None, n_splits: int = 1, chunk: int = 0,
@@ -1232,8 +1262,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
     value of every row by it.
     What only the vector kernel does (pages that are not blocked): v_dim, value heads of another width than the keys'
     (out is then [T, H * v_dim]); distance_bias = (a, b), two float32 tensors [H]: a[h] * ln(1 + b[h] * (i - j)) is taken
-    off the score of query position i and key position j; sink: the softmax has one more term of score 0 without a
-    value, i.e. 1 is added to its denominator."""
+    off the score of query position i and key position j; sink: the softmax has one more term without a value: True, of
+    score 0 (1 is added to its denominator); a float32 tensor [H], of that score per head (exp(sink[h]) is added)."""
     require_gpu()
     _dev(qkv, "qkv", dims=2)
     _dev(out, "out", qkv.dtype, 2)
@@ -1246,7 +1276,8 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         raise KernelError(f"attention: qkv {tuple(qkv.shape)} / out {tuple(out.shape)} do not fit H={H} hs={hs} v_dim={vd}")
     if vd % 2 or vd < 2 or vd > MAX_HEAD_DIM:
         raise KernelError(f"attention: value width {vd} is not supported (even, at most {MAX_HEAD_DIM})")
-    extras = vd != hs or distance_bias is not None or sink
+    sink_flag, sink_ptr = _sink_args(sink, H, "attention")
+    extras = vd != hs or distance_bias is not None or bool(sink_flag)
     if extras and layout == "blocked":
         raise KernelError("attention: another value width, a distance bias and a sink are the vector kernel's, which reads "
                           "pages with a row per position or transposed values")
@@ -1354,7 +1385,7 @@ def attention(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pag
         k_pages.data_ptr(), v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1],
         sl, tl, n_tiles, T, H, Hkv, hs, RT, GT, int(window), float(scale), int(n_splits), int(chunk),
         po, pm, int(vt), max_len_dev.data_ptr() if max_len_dev is not None else None, int(fold), vd,
-        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), _stream()),
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, sink_flag, sink_ptr, _stream()),
         "attention")
 
 
@@ -1465,8 +1496,8 @@ def attention_general_prompt(qkv: torch.Tensor, out: torch.Tensor, k_pages: torc
     _check(_fn("attn_mfma_general", "bn_attn_general_prompt")(
         qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * v_dim, k_pages.data_ptr(), v_pages.data_ptr(),
         block_table.data_ptr(), block_table.shape[1], tiles.data_ptr(), tiles.shape[0], H, Hkv, hs, v_dim, float(scale),
-        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), int(window),
-        _stream()), "attention_general_prompt")
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None,
+        *_sink_args(sink, H, "attention_general_prompt"), int(window), _stream()), "attention_general_prompt")
 
 
 def general_decode_plan(n_seqs: int, H: int, Hkv: int, max_len: int, window: int = 0):
@@ -1532,8 +1563,8 @@ def attention_general_decode(qkv: torch.Tensor, out: torch.Tensor, k_pages: torc
     _check(_fn("attn_mfma_general", "bn_attn_general_decode")(
         qkv.data_ptr(), _rows(qkv, "qkv"), out.data_ptr(), H * v_dim, k_pages.data_ptr(), v_pages.data_ptr(),
         block_table.data_ptr(), block_table.shape[1], seq_lens.data_ptr(), T, H, Hkv, hs, v_dim, float(scale),
-        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None, int(bool(sink)), int(window),
-        int(n_splits), int(chunk), part_o.data_ptr() if part_o is not None else None,
+        da.data_ptr() if da is not None else None, db.data_ptr() if db is not None else None,
+        *_sink_args(sink, H, "attention_general_decode"), int(window), int(n_splits), int(chunk), part_o.data_ptr() if part_o is not None else None,
         part_ml.data_ptr() if part_ml is not None else None,
         max_len_dev.data_ptr() if (max_len_dev is not None and n_splits > 1) else None, _stream()), "attention_general_decode")
 
@@ -1892,10 +1923,14 @@ def add_normed_rmsnorm(x: torch.Tensor, delta, out_weight: torch.Tensor, out_eps
 
 
 def latent_store(x: torch.Tensor, col: int, rank: int, weight: torch.Tensor, eps: float, positions, seq_index, block_table,
-                 k_pages: torch.Tensor, v_pages: torch.Tensor) -> None:
+                 k_pages: torch.Tensor, v_pages: torch.Tensor, *, rot_dims: int = 0, inv_freq: Optional[torch.Tensor] = None,
+                 rot_mult: float = 1.0) -> None:
     """Columns col .. col + rank of every row of x under an RMSNorm (weight [rank] float32, eps inside the root, float32
     arithmetic), stored at the row's position of its sequence's pages: as a key row ([pages, 1, PAGE, rank]) and into the
-    transposed value page ([pages, 1, rank, PAGE]).  Rows with position < 0 store nothing."""
+    transposed value page ([pages, 1, rank, PAGE]).  Rows with position < 0 store nothing.
+    rot_dims > 0: the next rot_dims columns of x are one more key part, not normed, dimension i turned with dimension
+    i + rot_dims / 2 by position * inv_freq[i] (cosine and sine times rot_mult); a key row is then rank + rot_dims wide
+    and holds it behind the latent, the value page stays rank wide."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(weight, "weight", torch.float32, 1)
@@ -1903,8 +1938,13 @@ def latent_store(x: torch.Tensor, col: int, rank: int, weight: torch.Tensor, eps
     _dev(seq_index, "seq_index", torch.int32, 1)
     _dev(block_table, "block_table", torch.int32, 2)
     T = x.shape[0]
-    _check_pages(k_pages, v_pages, 1, rank, x.dtype, True, False, rank)
-    if (col < 0 or x.shape[1] < col + rank or weight.numel() != rank or not weight.is_contiguous() or positions.numel() != T
+    rot_dims = int(rot_dims)
+    _check_pages(k_pages, v_pages, 1, rank + rot_dims, x.dtype, True, False, rank)
+    if rot_dims:
+        _dev(inv_freq, "inv_freq", torch.float32, 1)
+        if rot_dims % 2 or inv_freq.numel() != rot_dims // 2 or not inv_freq.is_contiguous():
+            raise KernelError(f"latent_store: {rot_dims} rotated dimensions need {rot_dims // 2} frequencies")
+    if (col < 0 or x.shape[1] < col + rank + rot_dims or weight.numel() != rank or not weight.is_contiguous() or positions.numel() != T
             or seq_index.numel() != T or not block_table.is_contiguous()):
         raise KernelError(f"latent_store: x {tuple(x.shape)} / columns {col}..{col + rank} / weight {tuple(weight.shape)} do not fit")
     if T == 0:
@@ -1912,16 +1952,38 @@ def latent_store(x: torch.Tensor, col: int, rank: int, weight: torch.Tensor, eps
     _check(_fn("latent", "bn_latent_store")(_code(x.dtype), x.data_ptr(), _rows(x, "x"), int(col), positions.data_ptr(),
                                             seq_index.data_ptr(), block_table.data_ptr(), block_table.shape[1],
                                             k_pages.data_ptr(), v_pages.data_ptr(), weight.data_ptr(), T, int(rank), float(eps),
+                                            rot_dims, inv_freq.data_ptr() if rot_dims else None, float(rot_mult),
                                             _stream()), "latent_store")
+
+
+def rope_heads(x: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, H: int, head_stride: int, offset: int,
+               rot_dims: int, mult: float = 1.0) -> None:
+    """In place on x [T, >= (H - 1) head_stride + offset + rot_dims]: in every head (head h starts at column
+    h * head_stride) the rot_dims columns from `offset` on are rotated, dimension i with dimension i + rot_dims / 2, by
+    position * inv_freq[i]; cosine and sine times `mult`.  Rows with position < 0 are left alone."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(positions, "positions", torch.int32, 1)
+    _dev(inv_freq, "inv_freq", torch.float32, 1)
+    T = x.shape[0]
+    if (rot_dims <= 0 or rot_dims % 2 or inv_freq.numel() != rot_dims // 2 or not inv_freq.is_contiguous() or offset < 0
+            or head_stride < offset + rot_dims or x.shape[1] < (H - 1) * head_stride + offset + rot_dims or positions.numel() != T):
+        raise KernelError(f"rope_heads: x {tuple(x.shape)} does not fit {H} heads of stride {head_stride} with {rot_dims} "
+                          f"rotated columns from {offset}")
+    if T:
+        _check(_fn("latent", "bn_rope_heads")(_code(x.dtype), x.data_ptr(), _rows(x, "x"), positions.data_ptr(),
+                                              inv_freq.data_ptr(), T, int(H), int(head_stride), int(offset), int(rot_dims),
+                                              float(mult), _stream()), "rope_heads")
 
 
 HEAD_LINEAR_MAX_IN = 1792          # the kernel stages 8 rows of a head's input as float32 beside its partial sums in 64 KB of shared memory
 
 
 def head_linear(x: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] = None, *,
-                allow_library: Optional[bool] = None) -> torch.Tensor:
+                allow_library: Optional[bool] = None, gate_per_head: bool = False) -> torch.Tensor:
     """A product per head: y[t, h, :] = x[t, h, :] . w[h] with x [T, H I] (rows contiguous), w [H, I, O] -> y [T, H O];
-    with `gate` [T, H O] (rows contiguous) y is multiplied by sigmoid(gate) element by element.  float32 accumulation.
+    with `gate` [T, H O] (rows contiguous) y is multiplied by sigmoid(gate) element by element, or, with gate_per_head,
+    head h of y by sigmoid of the one number gate[t, h] (gate [T, H]).  float32 accumulation.
     bf16 with more than SKINNY_ROWS rows goes to the library's batched product (allow_library as linear's), everything else
     to a kernel that reads every head's matrix once for 8 rows."""
     require_gpu()
@@ -1933,8 +1995,9 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] =
         raise KernelError(f"head_linear: x {tuple(x.shape)} and w {tuple(w.shape)} do not fit")
     if gate is not None:
         _dev(gate, "gate", x.dtype, 2)
-        if tuple(gate.shape) != (T, H * O):
-            raise KernelError(f"head_linear: gate {tuple(gate.shape)} is not [{T}, {H * O}]")
+        if tuple(gate.shape) != (T, H if gate_per_head else H * O):
+            raise KernelError(f"head_linear: gate {tuple(gate.shape)} is not [{T}, {H if gate_per_head else H * O}]")
+    group = O if gate_per_head else 1
     y = torch.empty((T, H * O), dtype=x.dtype, device=x.device)
     if T == 0:
         return y
@@ -1946,14 +2009,246 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, gate: Optional[torch.Tensor] =
         torch.bmm(xv, w, out=y.view(T, H, O).transpose(0, 1))
         if gate is not None:
             _check(_fn("latent", "bn_sigmoid_gate")(_code(y.dtype), y.data_ptr(), H * O, gate.data_ptr(), _rows(gate, "gate"),
-                                                    T, H * O, _stream()), "sigmoid_gate")
+                                                    group, T, H * O, _stream()), "sigmoid_gate")
         return y
     if I > HEAD_LINEAR_MAX_IN:
         raise KernelError(f"head_linear: a head's input of {I} values is above {HEAD_LINEAR_MAX_IN}")
     _check(_fn("latent", "bn_head_linear")(_code(x.dtype), x.data_ptr(), ldx, w.data_ptr(), y.data_ptr(), H * O,
                                            gate.data_ptr() if gate is not None else None,
-                                           _rows(gate, "gate") if gate is not None else 0, T, H, I, O, _stream()), "head_linear")
+                                           _rows(gate, "gate") if gate is not None else 0, group, T, H, I, O, _stream()),
+           "head_linear")
     return y
+
+
+# --------------------------------------------------------------------------------------
+# a residual of several streams and the norm without statistics (csrc/hyper.hip)
+# --------------------------------------------------------------------------------------
+
+HC_MAX_STREAMS = _build.header_constant("BN_HC_MAX_STREAMS", "hyper.hip")
+
+
+def hc_step(lanes_in: torch.Tensor, lanes_out: Optional[torch.Tensor], n: int, *, delta=None, mix=None, out_coef=None,
+            mult: float = 1.0, in_coef=None, norm=None, out_dtype=None, rows=None, read: bool = True):
+    """One pass over a residual of n streams.  lanes_in: [n, T, D] float32, or [T, D] read as every stream.  With `delta`
+    (a sublayer's output [T, D], float32 or bf16, or PartialSums) the streams are rebuilt first, x_t <- sum_s mix[s, t] x_s +
+    mult out_coef[t] delta, and stored in lanes_out [n, T, D] (which may be lanes_in; None: not stored).  Then, with `read`,
+    u = sum_s in_coef[s] x_s (in_coef None: the plain sum) is returned as [T or len(rows), D]: under norm = (weight, bias,
+    alpha) as tanh(alpha u) weight + bias in out_dtype, else u itself in out_dtype (float32 unless said).  rows: a choice of
+    rows (int32) for the result; the streams are then not stored.  mix [n, n], out_coef [n], in_coef [n] float32."""
+    require_gpu()
+    _dev(lanes_in, "lanes_in", torch.float32)
+    if lanes_in.dim() == 2:
+        T, D = lanes_in.shape
+        in_stride = 0
+    else:
+        if lanes_in.dim() != 3 or lanes_in.shape[0] != n:
+            raise KernelError(f"hc_step: {n} streams do not fit {tuple(lanes_in.shape)}")
+        _, T, D = lanes_in.shape
+        in_stride = T * D
+    if not lanes_in.is_contiguous() or not 1 <= n <= HC_MAX_STREAMS:
+        raise KernelError(f"hc_step: contiguous streams, at most {HC_MAX_STREAMS}")
+    if lanes_out is not None:
+        _dev(lanes_out, "lanes_out", torch.float32, 3)
+        if tuple(lanes_out.shape) != (n, T, D) or not lanes_out.is_contiguous() or rows is not None:
+            raise KernelError(f"hc_step: lanes_out {tuple(lanes_out.shape)} is not [{n}, {T}, {D}], or a choice of rows stores streams")
+    d_ptr, d_code, n_slabs = None, 0, 0
+    if delta is not None:
+        slabs = delta.slabs if isinstance(delta, PartialSums) else delta
+        _dev(slabs, "delta")
+        if tuple(slabs.shape[-2:]) != (T, D) or not slabs.is_contiguous() or slabs.dim() not in (2, 3):
+            raise KernelError(f"hc_step: delta {tuple(slabs.shape)} does not match the streams [{T}, {D}]")
+        n_slabs = slabs.shape[0] if slabs.dim() == 3 else 1
+        if slabs.dtype != torch.float32 and n_slabs != 1:
+            raise KernelError("hc_step: several slabs are float32 slabs")
+        d_ptr, d_code = slabs.data_ptr(), _code(slabs.dtype)
+        for t, nm, cnt in ((mix, "mix", n * n), (out_coef, "out_coef", n)):
+            _dev(t, nm, torch.float32)
+            if t.numel() != cnt or not t.is_contiguous():
+                raise KernelError(f"hc_step: {nm} must hold {cnt} float32 values")
+    if in_coef is not None:
+        _dev(in_coef, "in_coef", torch.float32, 1)
+        if in_coef.numel() != n or not in_coef.is_contiguous():
+            raise KernelError(f"hc_step: in_coef must hold {n} float32 values")
+    n_rows = T
+    if rows is not None:
+        _dev(rows, "rows", torch.int32, 1)
+        if not rows.is_contiguous():
+            raise KernelError("hc_step: rows must be contiguous")
+        n_rows = rows.numel()
+    w = b = alpha = None
+    if norm is not None:
+        w, b, alpha = norm
+        for t, nm, cnt in ((w, "norm weight", D), (b, "norm bias", D), (alpha, "norm alpha", 1)):
+            _dev(t, nm, torch.float32)
+            if t.numel() != cnt or not t.is_contiguous():
+                raise KernelError(f"hc_step: {nm} must hold {cnt} float32 values")
+    h = None
+    if read:
+        h = torch.empty((n_rows, D), dtype=out_dtype or torch.float32, device=lanes_in.device)
+    if n_rows == 0 or T == 0:
+        return h
+    _check(_fn("hyper", "bn_hc_step")(
+        d_code, _code(h.dtype) if h is not None else 0, lanes_in.data_ptr(), in_stride,
+        lanes_out.data_ptr() if lanes_out is not None else None, T * D, d_ptr, n_slabs, T * D,
+        mix.data_ptr() if delta is not None else None, out_coef.data_ptr() if delta is not None else None, float(mult),
+        in_coef.data_ptr() if in_coef is not None else None, w.data_ptr() if w is not None else None,
+        b.data_ptr() if b is not None else None, alpha.data_ptr() if alpha is not None else None,
+        h.data_ptr() if h is not None else None, rows.data_ptr() if rows is not None else None, n_rows, T, D, int(n),
+        _stream()), "hc_step")
+    return h
+
+
+def add_dyt_norm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, bias: torch.Tensor, alpha: torch.Tensor,
+                 out_dtype, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x (float32 [T, D]) += delta (out_dtype, optional; not with a choice of rows), then tanh(alpha x) * weight + bias of
+    all rows or of `rows`, in out_dtype.  weight, bias [D] and alpha (one number) float32 on the device."""
+    require_gpu()
+    _dev(x, "x", torch.float32, 2)
+    T, D = x.shape
+    for t, nm, cnt in ((weight, "weight", D), (bias, "bias", D), (alpha, "alpha", 1)):
+        _dev(t, nm, torch.float32)
+        if t.numel() != cnt or not t.is_contiguous():
+            raise KernelError(f"add_dyt_norm: {nm} must hold {cnt} float32 values")
+    if not x.is_contiguous() or (rows is not None and delta is not None):
+        raise KernelError("add_dyt_norm: x contiguous; a choice of rows leaves the stream as it is")
+    if delta is not None:
+        _dev(delta, "delta", out_dtype, 2)
+        if delta.shape != x.shape or not delta.is_contiguous():
+            raise KernelError(f"add_dyt_norm: delta {tuple(delta.shape)} does not match x {tuple(x.shape)}")
+    n = T
+    if rows is not None:
+        _dev(rows, "rows", torch.int32, 1)
+        n = rows.numel()
+    out = torch.empty((n, D), dtype=out_dtype, device=x.device)
+    if n:
+        _check(_fn("hyper", "bn_dyt_norm")(_code(out_dtype), x.data_ptr(), delta.data_ptr() if delta is not None else None,
+                                           weight.data_ptr(), bias.data_ptr(), alpha.data_ptr(), out.data_ptr(),
+                                           rows.data_ptr() if rows is not None else None, n, D, _stream()), "add_dyt_norm")
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# short convolutions and recurrences with a float32 state (csrc/conv_scans.hip)
+# --------------------------------------------------------------------------------------
+
+CONV_MAX_TAPS = _build.header_constant("BN_CONV_MAX_TAPS", "conv_scans.hip")
+GLA_MAX_DIM = _build.header_constant("GLA_MAX_DIM", "conv_scans.hip")
+
+
+def short_conv(x: torch.Tensor, col: int, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, positions,
+               seq_index, slot_ids, *, tiles=None, seq_lens=None, out_dtype=None) -> torch.Tensor:
+    """A causal convolution over time on C channels of x (columns col .. col + C): y_t = sum_j weight[:, j] u_(t - taps + 1 + j)
+    (+ bias), zeros before a sequence's first token.  weight [C, taps], bias [C] float32.  state: float32
+    [slots, >= (taps - 1) C] (a view that starts at this convolution's values): a sequence's inputs before the step's
+    first token, oldest first; read for a step's first tokens and left holding the step's last inputs.  tiles (one a
+    sequence) in a prompt step, seq_lens in a decode step.  Returns y [T, C] in out_dtype (x's unless said)."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(weight, "weight", torch.float32, 2)
+    T = x.shape[0]
+    C, taps = weight.shape
+    if not weight.is_contiguous() or not 1 <= taps <= CONV_MAX_TAPS or col < 0 or x.shape[1] < col + C:
+        raise KernelError(f"short_conv: x {tuple(x.shape)} / columns {col}..{col + C} / weight {tuple(weight.shape)} do not fit "
+                          f"(at most {CONV_MAX_TAPS} taps)")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32, 1)
+        if bias.numel() != C or not bias.is_contiguous():
+            raise KernelError(f"short_conv: bias must hold {C} float32 values")
+    stride = _state_rows(state, (taps - 1) * C, "short_conv")
+    for t, nm in ((positions, "positions"), (seq_index, "seq_index")):
+        _dev(t, nm, torch.int32, 1)
+        if t.numel() != T or not t.is_contiguous():
+            raise KernelError(f"short_conv: {nm} must hold one int32 per row")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    tl, n_seqs, sl = _seq_args(tiles, seq_lens, "short_conv")
+    if tl is None and n_seqs != T:
+        raise KernelError("short_conv: a decode step has one row a sequence")
+    y = torch.empty((T, C), dtype=out_dtype or x.dtype, device=x.device)
+    if T and n_seqs:
+        _check(_fn("conv_scans", "bn_short_conv")(
+            _code(x.dtype), _code(y.dtype), x.data_ptr(), _rows(x, "x"), int(col), y.data_ptr(), C, weight.data_ptr(),
+            bias.data_ptr() if bias is not None else None, state.data_ptr(), stride, positions.data_ptr(), seq_index.data_ptr(),
+            slot_ids.data_ptr(), tl, sl, n_seqs, T, C, taps, _stream()), "short_conv")
+    return y
+
+
+def lru_gates(u: torch.Tensor, wa_t: torch.Tensor, ba: torch.Tensor, wi_t: torch.Tensor, bi: torch.Tensor,
+              c_neg: torch.Tensor):
+    """The operands of a real-gated linear recurrent unit from its input u [T, W] float32: u in `blocks` equal parts, in
+    part b r = sigmoid(u_b . wa_t[b] + ba), i = sigmoid(u_b . wi_t[b] + bi) (wa_t, wi_t [blocks, in, out] float32, the
+    biases [W]); a = exp(c_neg r) (c_neg [W], the channel's -8 softplus(lam)).  Returns (a, sqrt(1 - a^2) i u), float32
+    [T, W] each.  All of it in float32."""
+    require_gpu()
+    _dev(u, "u", torch.float32, 2)
+    T, W = u.shape
+    _dev(wa_t, "wa_t", torch.float32, 3)
+    _dev(wi_t, "wi_t", torch.float32, 3)
+    blocks = wa_t.shape[0]
+    bw = W // max(blocks, 1)
+    if (blocks < 1 or W % blocks or tuple(wa_t.shape) != (blocks, bw, bw) or tuple(wi_t.shape) != (blocks, bw, bw)
+            or not (u.is_contiguous() and wa_t.is_contiguous() and wi_t.is_contiguous()) or bw * 32 > 64 * 1024):
+        raise KernelError(f"lru_gates: u {tuple(u.shape)} and gate matrices {tuple(wa_t.shape)} / {tuple(wi_t.shape)} do not fit")
+    for t, nm in ((ba, "ba"), (bi, "bi"), (c_neg, "c_neg")):
+        _dev(t, nm, torch.float32, 1)
+        if t.numel() != W or not t.is_contiguous():
+            raise KernelError(f"lru_gates: {nm} must hold {W} float32 values")
+    a = torch.empty((T, W), dtype=torch.float32, device=u.device)
+    b = torch.empty((T, W), dtype=torch.float32, device=u.device)
+    if T:
+        _check(_fn("conv_scans", "bn_lru_gates")(u.data_ptr(), wa_t.data_ptr(), ba.data_ptr(), wi_t.data_ptr(), bi.data_ptr(),
+                                                 c_neg.data_ptr(), a.data_ptr(), b.data_ptr(), T, W, blocks, _stream()), "lru_gates")
+    return a, b
+
+
+def lru_scan(a: torch.Tensor, b: torch.Tensor, y_pre: torch.Tensor, state: torch.Tensor, slot_ids, *, tiles=None,
+             seq_lens=None) -> torch.Tensor:
+    """S <- a_t S + b_t per channel over every sequence's tokens (a, b [T, W] float32; S from the sequence's state row,
+    zeros at position 0, left there afterwards), the result times gelu_tanh(y_pre) (y_pre [T, W] in the activations'
+    type, which is the result's)."""
+    require_gpu()
+    _dev(a, "a", torch.float32, 2)
+    _dev(b, "b", torch.float32, 2)
+    _dev(y_pre, "y_pre", dims=2)
+    T, W = a.shape
+    if tuple(b.shape) != (T, W) or tuple(y_pre.shape) != (T, W) or not (a.is_contiguous() and b.is_contiguous()):
+        raise KernelError(f"lru_scan: a {tuple(a.shape)}, b {tuple(b.shape)}, y_pre {tuple(y_pre.shape)} do not fit")
+    stride = _state_rows(state, W, "lru_scan")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    tl, n_seqs, sl = _seq_args(tiles, seq_lens, "lru_scan")
+    out = torch.empty((T, W), dtype=y_pre.dtype, device=a.device)
+    if T and n_seqs:
+        _check(_fn("conv_scans", "bn_lru_scan")(_code(y_pre.dtype), a.data_ptr(), b.data_ptr(), y_pre.data_ptr(), _rows(y_pre, "y_pre"),
+                                                out.data_ptr(), state.data_ptr(), stride, tl, n_seqs, sl, slot_ids.data_ptr(), W,
+                                                _stream()), "lru_scan")
+    return out
+
+
+def gla_supported(dk: int, dv: int) -> bool:
+    return bool(_fn("conv_scans", "bn_gla_supports")(int(dk), int(dv)))
+
+
+def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, state: torch.Tensor, slot_ids, H: int,
+             dk: int, dv: int, q_scale: float, inv_tau: float, *, tiles=None, seq_lens=None) -> torch.Tensor:
+    """Gated linear attention over every sequence's tokens: per head S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T (q_scale q_t)
+    with alpha = sigmoid(z)^inv_tau per key channel.  x [T, ld] holds q at q_col, k at k_col (heads of dk) and v at v_col
+    (heads of dv); z [T, H dk] float32.  state: float32 [slots, >= H dk dv], a head's matrix [dk, dv] row-major; zeros at
+    position 0.  Returns o [T, H dv] float32."""
+    require_gpu()
+    _dev(x, "x", dims=2)
+    _dev(z, "z", torch.float32, 2)
+    T = x.shape[0]
+    if (not gla_supported(dk, dv) or x.shape[1] < max(q_col + H * dk, k_col + H * dk, v_col + H * dv) or min(q_col, k_col, v_col) < 0
+            or tuple(z.shape) != (T, H * dk) or not z.is_contiguous()):
+        raise KernelError(f"gla_scan: x {tuple(x.shape)} / z {tuple(z.shape)} do not fit H={H} dk={dk} dv={dv} (dk at most {GLA_MAX_DIM})")
+    stride = _state_rows(state, H * dk * dv, "gla_scan")
+    _dev(slot_ids, "slot_ids", torch.int32, 1)
+    tl, n_seqs, sl = _seq_args(tiles, seq_lens, "gla_scan")
+    o = torch.empty((T, H * dv), dtype=torch.float32, device=x.device)
+    if T and n_seqs:
+        _check(_fn("conv_scans", "bn_gla_scan")(_code(x.dtype), x.data_ptr(), _rows(x, "x"), int(q_col), int(k_col), int(v_col),
+                                                z.data_ptr(), o.data_ptr(), state.data_ptr(), stride, tl, n_seqs, sl,
+                                                slot_ids.data_ptr(), H, dk, dv, float(q_scale), float(inv_tau), _stream()), "gla_scan")
+    return o
 
 
 MOE_MAX_EXPERTS = _build.header_constant("MOE_MAX_EXPERTS", "moe.hip")
@@ -1963,9 +2258,9 @@ MOE_SCORINGS = {"sigmoid": _build.header_constant("MOE_SCORE_SIGMOID", "moe.hip"
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = "sigmoid", renormalize: bool = False, *,
               choice_bias: Optional[torch.Tensor] = None, weight_floor: float = 0.0, weight_scale: float = 1.0,
-              gate: Optional[torch.Tensor] = None):
-    """(ids [T, top_k] int32, weights [T, top_k] float32): router logits z = router . h in float32 (router [E, D]
-    float32, h in the activations' type), scores sigmoid(z) or softmax(z) over the experts, the top_k largest in
+              gate: Optional[torch.Tensor] = None, logit_bias: Optional[torch.Tensor] = None):
+    """(ids [T, top_k] int32, weights [T, top_k] float32): router logits z = router . h (+ logit_bias [E] float32) in
+    float32 (router [E, D] float32, h in the activations' type), scores sigmoid(z) or softmax(z) over the experts, the top_k largest in
     descending order (ties: the lower index); renormalize divides the chosen scores by their sum (+ weight_floor);
     weight_scale multiplies the weights.  choice_bias [E] float32: the experts are chosen by score + bias, the weights
     stay the plain scores.  gate [D] float32: a third result [T] float32, sigmoid(gate . h), a shared expert's gate."""
@@ -1979,7 +2274,7 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = 
     if router.shape[1] != D or not router.is_contiguous() or not 1 <= top_k <= E or E > MOE_MAX_EXPERTS or D > 16384:
         raise KernelError(f"moe_route: h {tuple(h.shape)}, router {tuple(router.shape)}, top_k {top_k} do not fit "
                           f"(at most {MOE_MAX_EXPERTS} experts, 16,384 columns)")
-    for t, nm, n in ((choice_bias, "choice_bias", E), (gate, "gate", D)):
+    for t, nm, n in ((choice_bias, "choice_bias", E), (gate, "gate", D), (logit_bias, "logit_bias", E)):
         if t is not None:
             _dev(t, nm, torch.float32, 1)
             if t.numel() != n or not t.is_contiguous():
@@ -1994,7 +2289,8 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, top_k: int, scoring: str = 
                                           wts.data_ptr(), T, D, E, int(top_k), MOE_SCORINGS[scoring], int(bool(renormalize)),
                                           choice_bias.data_ptr() if choice_bias is not None else None, float(weight_floor),
                                           float(weight_scale), gate.data_ptr() if gate is not None else None,
-                                          gate_out.data_ptr() if gate is not None else None, _stream()), "moe_route")
+                                          gate_out.data_ptr() if gate is not None else None,
+                                          logit_bias.data_ptr() if logit_bias is not None else None, _stream()), "moe_route")
     return (ids, wts) if gate is None else (ids, wts, gate_out)
 
 

@@ -24,7 +24,12 @@ split-half or in neighbouring pairs, over the first rope_dims dimensions) and ta
   q_temp_coef, q_temp_every   the query at position p times 1 + coef * ln(floor((p + 1) / every) + 1)
   distance_bias  tensors dist_a, dist_b [heads]: dist_a[h] * ln(1 + dist_b[h] * (i - j)) is taken off the score of
                  query i and key j
-  sink           the softmax has one more term of score 0 and no value: p_j = exp(s_j) / (1 + sum exp(s))
+  sink           the softmax has one more term of score 0 and no value: p_j = exp(s_j) / (1 + sum exp(s)); "learned": the
+                 term's score is a number per head (tensor sink [heads]): p_j = exp(s_j) / (exp(sink_h) + sum exp(s))
+  conv_taps      a short causal convolution over time on every channel of the query and key projections, directly behind the
+                 projection (tensors q_conv [heads head_dim, taps], k_conv [kv heads head_dim, taps], no bias; the last
+                 column meets the current token, zeros before a sequence's first token); with value_is_key the values are
+                 the keys as they leave it.  A sequence's last taps - 1 projected rows are a state beside its pages.
   value_is_key   there is no value projection: kv head g's value is its key projection as projected, before the key's norm
                  and rotation (the tensor wv does not exist; the value heads are as wide as the key heads)
 """
@@ -33,7 +38,7 @@ from __future__ import annotations
 import torch
 
 from .. import ops
-from .base import MIXERS, POSITION_ENCODINGS, CacheNeed, KVNeed, ParamSpec, Part, PartSpec
+from .base import MIXERS, POSITION_ENCODINGS, CacheNeed, KVNeed, ParamSpec, Part, PartSpec, StateNeed
 from .linear import Linear, upload
 
 
@@ -49,7 +54,8 @@ class Attention(Part):
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  position: PartSpec, window: int = 0, bias: bool = False, v_head_dim: int = 0,
                  qk_norm_eps: float | None = None, q_temp_coef: float = 0.0, q_temp_every: int = 0,
-                 distance_bias: bool = False, sink: bool = False, qk_norm_span: str = "head", value_is_key: bool = False):
+                 distance_bias: bool = False, sink=False, qk_norm_span: str = "head", value_is_key: bool = False,
+                 conv_taps: int = 0):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
         if head_dim % 2 or head_dim < 2 or head_dim > ops.MAX_HEAD_DIM:
@@ -65,7 +71,12 @@ class Attention(Part):
             raise ValueError(f"attention: values that are the keys are as wide as the keys, got {self.vd} and {self.hs}")
         self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.q_temp_coef, self.q_temp_every = float(q_temp_coef), int(q_temp_every)
-        self.distance_bias, self.sink = bool(distance_bias), bool(sink)
+        if sink not in (False, True, "learned"):
+            raise ValueError(f"attention: sink {sink!r} is neither False, True nor 'learned'")
+        self.distance_bias, self.sink, self.sink_learned = bool(distance_bias), bool(sink), sink == "learned"
+        self.conv_taps = int(conv_taps)
+        if self.conv_taps < 0 or self.conv_taps > ops.CONV_MAX_TAPS:
+            raise ValueError(f"attention: conv_taps {conv_taps} (at most {ops.CONV_MAX_TAPS})")
         if qk_norm_span not in ("head", "projection"):
             raise ValueError(f"attention: qk_norm_span {qk_norm_span!r} is neither 'head' nor 'projection'")
         self.norm_projection = qk_norm_span == "projection"
@@ -73,7 +84,7 @@ class Attention(Part):
             raise ValueError("attention: a norm over the whole projection needs qk_norm_eps")
         self.general = (self.vd != self.hs or self.qk_norm_eps is not None or self.q_temp_every > 0
                         or self.distance_bias or self.sink or getattr(self.position, "interleaved", False)
-                        or self.value_is_key)
+                        or self.value_is_key or self.conv_taps > 0)
         if self.general:
             if self.vd % 2 or self.vd < 2 or self.vd > ops.MAX_HEAD_DIM:
                 raise ValueError(f"attention: v_head_dim {self.vd} is not supported by the kernels (even, at most {ops.MAX_HEAD_DIM})")
@@ -81,7 +92,7 @@ class Attention(Part):
                 raise ValueError("attention: head norms, a query temperature, a distance bias, a sink, a rotation in neighbouring "
                                  "pairs, values of another width or values that are the keys come without projection biases")
             self.takes_deferred_norm = self.gives_lazy_delta = False
-        self.q_norm = self.k_norm = self.dist_a = self.dist_b = None
+        self.q_norm = self.k_norm = self.dist_a = self.dist_b = self.sink_values = self.conv_w = None
 
     @property
     def q_dim(self):
@@ -101,6 +112,10 @@ class Attention(Part):
             t.update({"q_norm": ParamSpec((nq,), "ones"), "k_norm": ParamSpec((nk,), "ones")})
         if self.distance_bias:
             t.update({"dist_a": ParamSpec((self.H,), "normal"), "dist_b": ParamSpec((self.H,), "ones")})
+        if self.sink_learned:
+            t["sink"] = ParamSpec((self.H,), "normal")
+        if self.conv_taps:
+            t.update({"q_conv": ParamSpec((self.q_dim, self.conv_taps)), "k_conv": ParamSpec((self.kv_dim, self.conv_taps))})
         if self.has_bias:
             t.update({"bq": ParamSpec((self.q_dim,), "normal"), "bk": ParamSpec((self.kv_dim,), "normal"),
                       "bv": ParamSpec((self.kv_dim,), "normal"), "bo": ParamSpec((self.hidden,), "normal")})
@@ -120,6 +135,10 @@ class Attention(Part):
             self.q_norm, self.k_norm = (upload(tensors[n], device, torch.float32) for n in ("q_norm", "k_norm"))
         if self.distance_bias:
             self.dist_a, self.dist_b = (upload(tensors[n], device, torch.float32) for n in ("dist_a", "dist_b"))
+        if self.sink_learned:
+            self.sink_values = upload(tensors["sink"], device, torch.float32)
+        if self.conv_taps:
+            self.conv_w = torch.cat([upload(tensors[n], device, torch.float32) for n in ("q_conv", "k_conv")], dim=0).contiguous()
 
     def linears(self):
         return [self.qkv, self.o]
@@ -127,7 +146,10 @@ class Attention(Part):
     def cache_need(self) -> CacheNeed:
         if self.general:                  # keys a row per position, values transposed inside a page, in both types: what the
             # vector kernel and the general prompt kernel on the matrix cores both read
-            return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window, v_head_dim=self.vd, v_layout="transposed"))
+            state = None
+            if self.conv_taps > 1:        # the projected query and key rows of the last taps - 1 positions, float32
+                state = StateNeed(((self.conv_taps - 1) * (self.q_dim + self.kv_dim),), torch.float32, device_addressed=True)
+            return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window, v_head_dim=self.vd, v_layout="transposed"), state=state)
         return CacheNeed(kv=KVNeed(self.Hkv, self.hs, self.window))
 
     def wants_deferred_norm(self, ctx, rows: int) -> bool:
@@ -152,6 +174,15 @@ class Attention(Part):
         else:
             qkv = torch.empty((h.shape[0], width), dtype=h.dtype, device=h.device)
             qkv[:, :self.q_dim] = self.qkv(h, rows=slice(0, self.q_dim))
+        if self.conv_taps:
+            if not kv.writes:
+                raise ValueError("attention: a convolution on the projections needs the layer's own keys")
+            seqs = dict(seq_lens=ctx.seq_lens) if ctx.is_decode else dict(tiles=ctx.tiles(ops.SEQUENCE_TILE))
+            qk = ops.short_conv(qkv, 0, self.conv_w, None, kv.state, ctx.positions, ctx.seq_index, ctx.slot_ids, **seqs)
+            if self.value_is_key:
+                qkv = qk
+            else:
+                qkv[:, :self.q_dim + self.kv_dim].copy_(qk)
         ops.qk_norm_store(qkv, ctx.positions, H, Hkv, hs, v_dim=vd, q_weight=self.q_norm, k_weight=self.k_norm,
                           eps=self.qk_norm_eps or 0.0, temp_coef=self.q_temp_coef, temp_every=self.q_temp_every,
                           norm_projection=self.norm_projection, inv_freq=self.position.inv_freq,
@@ -168,7 +199,7 @@ class Attention(Part):
             ops.attention_general_decode(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, ctx.seq_lens, H, Hkv, hs, vd, self.scale,
                                          window=self.window, n_splits=n_splits, chunk=chunk,
                                          max_len_dev=ctx.max_len_dev if follows and n_splits > 1 else None,
-                                         distance_bias=bias, sink=self.sink)
+                                         distance_bias=bias, sink=self._sink())
         elif ctx.is_decode:
             if not self.window:
                 n_splits, chunk = ops.decode_splits(ctx.n_rows, H, Hkv, kv.max_len, h.dtype, target_wgs=ops.VECTOR_DECODE_TARGET_WGS)
@@ -182,17 +213,20 @@ class Attention(Part):
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
                           seq_lens=ctx.seq_lens, n_splits=n_splits, chunk=chunk,
                           max_len_dev=ctx.max_len_dev if n_splits > 1 and not self.window else None, v_transposed=True, blocked=False,
-                          v_dim=vd, distance_bias=bias, sink=self.sink)
+                          v_dim=vd, distance_bias=bias, sink=self._sink())
         elif on_matrix_cores:
             ops.attention_general_prompt(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, vd, self.scale,
-                                         ctx.tiles(ops.GENERAL_PROMPT_TILE), distance_bias=bias, sink=self.sink,
+                                         ctx.tiles(ops.GENERAL_PROMPT_TILE), distance_bias=bias, sink=self._sink(),
                                          window=self.window)
         else:
             _, _, qt = ops.attention_row_shape(H, Hkv, False)
             ops.attention(qkv, out, kv.k_pages, kv.v_pages, kv.block_table, H, Hkv, hs, self.scale, window=self.window,
                           tiles=ctx.tiles(qt), qt=qt, v_transposed=True, blocked=False, v_dim=vd, distance_bias=bias,
-                          sink=self.sink)
+                          sink=self._sink())
         return self.o(out)
+
+    def _sink(self):
+        return self.sink_values if self.sink_learned else self.sink
 
     def forward(self, h, ctx, kv, lazy_ok: bool = False):
         if self.general:

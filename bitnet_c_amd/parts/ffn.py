@@ -44,6 +44,38 @@ class DenseFFN(Part):
         return self.down.lazy(a) if lazy_ok else self.down(a)
 
 
+@FEED_FORWARDS.register("gated_clamped")
+class ClampedGatedFFN(Part):
+    """A gated feed-forward whose unit bounds its arguments: down(g' sigmoid(slope g') (u' + shift)) with g' = min(W_gate h,
+    limit), u' = clamp(W_up h, -limit, limit).  Gate and up rows are stacked ([F gate rows; F up rows]): one product, then
+    the unit's kernel (ops.gated_unit, the one a mixture's shared expert uses), then the last product."""
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+    gives_lazy_delta = True         # forward(..., lazy_ok=True) may return a LazyDelta
+
+    def __init__(self, hidden: int, intermediate: int, limit: float, slope: float = 1.702, shift: float = 1.0):
+        self.hidden, self.F = int(hidden), int(intermediate)
+        self.unit = ops.ClampedUnit(float(limit), float(slope), float(shift))
+        self.gate_up, self.down = Linear(), Linear()
+
+    def tensors(self):
+        return {"w_gate": ParamSpec((self.F, self.hidden)), "w_up": ParamSpec((self.F, self.hidden)),
+                "w_down": ParamSpec((self.hidden, self.F))}
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("w_gate", "w_up")], dim=0).contiguous()
+        self.gate_up.load(w, None, device, dtype)
+        self.down.load(tensors["w_down"], None, device, dtype)
+
+    def linears(self):
+        return [self.gate_up, self.down]
+
+    def forward(self, h, ctx, lazy_ok: bool = False):
+        if isinstance(h, ops.DeferredNorm):
+            h = h.materialize()
+        act = ops.gated_unit(self.gate_up(h), self.unit)
+        return self.down.lazy(act) if lazy_ok else self.down(act)
+
+
 @FEED_FORWARDS.register("gated")
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(Part):

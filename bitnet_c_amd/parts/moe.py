@@ -14,6 +14,9 @@ Options beside that form, each off by default:
   choice_bias      a tensor `correction` [n_experts]: the experts with the largest score + correction are chosen; the
                    weights stay the plain scores
   weight_floor     joins the sum that `renormalize` divides by;  weight_scale multiplies the weights
+  gated            (without expert_limit) the experts are plain gated units W_down,e (act(W_gate,e x) * (W_up,e x)) with
+                   act = silu: the unit above without bounds, slope 1 and shift 0
+  router_bias      a tensor `router_bias` [n_experts] added to the logits themselves, before scoring and choice
   shared_intermediate (with shared_limit)   one more gated unit of that width that every token runs (shared.w_gate,
                    shared.w_up, shared.w_down), its output times sigmoid(shared.gate . h), one number per token
 
@@ -40,7 +43,8 @@ class MoEFFN(Part):
     def __init__(self, hidden: int, n_experts: int, top_k: int, intermediate: int, activation: str = "relu2",
                  scoring: str = "sigmoid", renormalize: bool = False, weight_on: str = "input", expert_limit: float = 0.0,
                  gate_slope: float = 1.702, up_shift: float = 1.0, choice_bias: bool = False, weight_floor: float = 0.0,
-                 weight_scale: float = 1.0, shared_intermediate: int = 0, shared_limit: float = 0.0):
+                 weight_scale: float = 1.0, shared_intermediate: int = 0, shared_limit: float = 0.0, gated: bool = False,
+                 router_bias: bool = False):
         if activation not in ops.UNARY_ACTIVATIONS:
             raise ValueError(f"moe: unknown activation {activation!r}; known: {sorted(ops.UNARY_ACTIVATIONS)}")
         if scoring not in ops.MOE_SCORINGS:
@@ -53,6 +57,11 @@ class MoEFFN(Part):
         self.activation, self.scoring, self.renormalize = activation, scoring, bool(renormalize)
         self.weight_on_input = weight_on == "input"
         self.unit = ops.ClampedUnit(float(expert_limit), float(gate_slope), float(up_shift)) if expert_limit else None
+        if gated and self.unit is None:
+            if activation != "silu":
+                raise ValueError(f"moe: gated experts without bounds take the activation 'silu', got {activation!r}")
+            self.unit = ops.ClampedUnit(float("inf"), 1.0, 0.0)
+        self.has_router_bias = bool(router_bias)
         self.has_choice_bias, self.weight_floor, self.weight_scale = bool(choice_bias), float(weight_floor), float(weight_scale)
         if self.weight_floor < 0 or not self.weight_scale > 0:
             raise ValueError(f"moe: weight_floor {weight_floor} must not be negative and weight_scale {weight_scale} be positive")
@@ -61,12 +70,14 @@ class MoEFFN(Part):
             raise ValueError("moe: a shared expert has a width and a limit, or there is none")
         self.shared_unit = ops.ClampedUnit(float(shared_limit), float(gate_slope), float(up_shift)) if self.Fs else None
         self.shared_up, self.shared_down = Linear(), Linear()
-        self.router = self.w_up = self.w_down = self.choice_bias = self.shared_gate = None
+        self.router = self.w_up = self.w_down = self.choice_bias = self.shared_gate = self.router_bias = None
 
     def tensors(self):
         t = {"router": ParamSpec((self.E, self.hidden))}
         if self.has_choice_bias:
             t["correction"] = ParamSpec((self.E,), "normal")
+        if self.has_router_bias:
+            t["router_bias"] = ParamSpec((self.E,), "normal")
         for e in range(self.E):
             if self.unit is not None:
                 t[f"e{e}.w_gate"] = ParamSpec((self.F, self.hidden))
@@ -89,6 +100,8 @@ class MoEFFN(Part):
             self.w_down[e].copy_(upload(tensors[f"e{e}.w_down"], device, dtype))
         if self.has_choice_bias:
             self.choice_bias = upload(tensors["correction"], device, torch.float32)
+        if self.has_router_bias:
+            self.router_bias = upload(tensors["router_bias"], device, torch.float32)
         if self.Fs:
             w = torch.cat([upload(tensors[n], device, dtype) for n in ("shared.w_gate", "shared.w_up")], dim=0).contiguous()
             self.shared_up.load(w, None, device, dtype)
@@ -102,7 +115,8 @@ class MoEFFN(Part):
         if isinstance(h, ops.DeferredNorm):
             h = h.materialize()
         routed = ops.moe_route(h, self.router, self.K, self.scoring, self.renormalize, choice_bias=self.choice_bias,
-                               weight_floor=self.weight_floor, weight_scale=self.weight_scale, gate=self.shared_gate)
+                               weight_floor=self.weight_floor, weight_scale=self.weight_scale, gate=self.shared_gate,
+                               logit_bias=self.router_bias)
         ids, wts = routed[0], routed[1]
         experts = ops.moe_experts_grouped if ops.moe_grouped_supported(h.shape[0], self.hidden, self.F, h.dtype) else ops.moe_experts
         y = experts(h, self.w_up, self.w_down, ids, wts, self.activation, self.weight_on_input, gated=self.unit,

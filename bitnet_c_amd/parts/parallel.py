@@ -3,15 +3,18 @@ width (plain weights "left_out" / "right_out", eps inside the root), and the res
 
     y = 1/2 (rmsnorm(left(h)) * w_left + rmsnorm(right(h)) * w_right)
 
-The two are any registered mixers; between them they may keep one set of keys and values and one state of fixed size
-(the cache gives an entry of the schedule one of each), which is what an attention beside a recurrence needs.
+The two are any registered mixers; between them they may keep one set of keys and values (the cache gives an entry of
+the schedule one).  Each may keep a state of fixed size: two float32 states addressed by the step's slot ids lie side by
+side in the entry's one state row, the left mixer's first, and each mixer sees its own columns.
 """
 from __future__ import annotations
+
+import dataclasses
 
 import torch
 
 from .. import ops
-from .base import MIXERS, CacheNeed, ParamSpec, Part, PartSpec
+from .base import MIXERS, CacheNeed, ParamSpec, Part, PartSpec, StateNeed
 from .linear import upload
 
 
@@ -21,8 +24,14 @@ class ParallelMixer(Part):
         self.hidden, self.eps = int(hidden), float(eps)
         self.left, self.right = MIXERS.build(left), MIXERS.build(right)
         needs = [self.left.cache_need(), self.right.cache_need()]
-        if sum(n.kv is not None for n in needs) > 1 or sum(n.state is not None for n in needs) > 1:
-            raise ValueError("parallel mixer: its two mixers may keep one set of keys and values and one state between them")
+        if sum(n.kv is not None for n in needs) > 1:
+            raise ValueError("parallel mixer: its two mixers may keep one set of keys and values between them")
+        self.state_split = None                  # floats of the left mixer's state when both keep one
+        if all(n.state is not None for n in needs):
+            for n in needs:
+                if len(n.state.shape) != 1 or n.state.dtype != torch.float32:
+                    raise ValueError("parallel mixer: two states share a row only as flat float32 states")
+            self.state_split = int(needs[0].state.shape[0])
         self.w_left = self.w_right = None
 
     @property
@@ -48,9 +57,17 @@ class ParallelMixer(Part):
 
     def cache_need(self) -> CacheNeed:
         a, b = self.left.cache_need(), self.right.cache_need()
-        return CacheNeed(kv=a.kv or b.kv, state=a.state or b.state)
+        state = a.state or b.state
+        if self.state_split is not None:
+            state = StateNeed((a.state.shape[0] + b.state.shape[0],), torch.float32,
+                              device_addressed=a.state.device_addressed and b.state.device_addressed)
+        return CacheNeed(kv=a.kv or b.kv, state=state)
 
     def forward(self, h, ctx, kv):
-        a = self.left.forward(h, ctx, kv)
-        b = self.right.forward(h, ctx, kv)
+        kv_a = kv_b = kv
+        if self.state_split is not None:
+            kv_a = dataclasses.replace(kv, state=kv.state[:, :self.state_split])
+            kv_b = dataclasses.replace(kv, state=kv.state[:, self.state_split:])
+        a = self.left.forward(h, ctx, kv_a)
+        b = self.right.forward(h, ctx, kv_b)
         return ops.rmsnorm_mean(a, self.w_left, b, self.w_right, self.eps)

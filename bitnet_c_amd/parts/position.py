@@ -10,6 +10,11 @@ frequencies on this path; the "llama3" rescaling is written from its definition:
 wavelengths below orig/high_freq_factor stay, those above orig/low_freq_factor are
 divided by `factor`, those between are interpolated linearly in orig/wavelength.
 
+The "yarn" rescaling (keys factor, original, fast, slow): with d(t) = dims ln(original / (2 pi t)) / (2 ln theta),
+lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the
+frequency is f_i / factor where r_i = 1, f_i where r_i = 0 and r_i f_i / factor + (1 - r_i) f_i between; every cosine and
+sine is also multiplied by 0.1 ln(factor) + 1 (rope_magnitude), which a mixer that rotates applies itself.
+
 "none": no encoding; K and V are stored as they are.
 """
 from __future__ import annotations
@@ -35,9 +40,27 @@ def rope_frequencies(rope_dims: int, theta: float, scaling: dict | None = None) 
             smooth = (orig / wavelen - low) / (high - low)
             mid = (1.0 - smooth) * f / factor + smooth * f
             f = torch.where(wavelen < orig / high, f, torch.where(wavelen > orig / low, f / factor, mid))
+        elif kind == "yarn":
+            factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+            def corr(turns):
+                return rope_dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(theta)))
+
+            lo = max(math.floor(corr(float(scaling["fast"]))), 0)
+            hi = min(math.ceil(corr(float(scaling["slow"]))), rope_dims - 1)
+            ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+            f = f / factor * ramp + f * (1.0 - ramp)
         elif kind not in (None, "default"):
             raise ValueError(f"position encoding: unknown frequency scaling {kind!r}")
     return f.to(torch.float32)
+
+
+def rope_magnitude(scaling: dict | None = None) -> float:
+    """What multiplies every cosine and sine of a rotation with this frequency scaling: 0.1 ln(factor) + 1 for "yarn",
+    else 1."""
+    if scaling and scaling.get("rope_type") == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 class PositionEncoding(Part):

@@ -188,3 +188,133 @@ class Lightning(Part):
                                **_sequences(ctx))
         y = ops.row_norm_gate(o, x[:, self.g_col:], self.norm, self.eps, self.gate_activation)
         return self.o(y)
+
+
+@MIXERS.register("gla")
+class GatedLinearAttention(Part):
+    """Linear attention with a matrix state per head and a decay per key channel that depends on the token
+    (csrc/conv_scans.hip):
+        q = W_q h / sqrt(head_dim), k = W_k h   heads x head_dim;   v = W_v h   heads x v_head_dim
+        alpha = sigmoid(W_a2 (W_a1 h) + b)^(1 / tau)                 heads x head_dim, float32
+        S <- diag(alpha_t) S + k_t v_t^T;   o_t = S^T q_t            the decay acts on the rows of the key channels
+        y = W_o (o / rms_head(o) * norm * silu(W_g h))               every head by its own root mean square, norm [v_head_dim]
+    The decay's low-rank input rides in the stacked projection; its logits leave their product as float32."""
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+
+    def __init__(self, hidden: int, n_heads: int, head_dim: int, v_head_dim: int, decay_rank: int, tau: float, eps: float):
+        self.hidden, self.H, self.hs, self.vd = int(hidden), int(n_heads), int(head_dim), int(v_head_dim) or int(head_dim)
+        self.rank, self.tau, self.eps = int(decay_rank), float(tau), float(eps)
+        if not ops.gla_supported(self.hs, self.vd):
+            raise ValueError(f"gla: head_dim {self.hs} is not supported by the kernel (at most {ops.GLA_MAX_DIM})")
+        if not self.tau > 0 or self.rank < 1:
+            raise ValueError(f"gla: tau {tau} must be positive and the decay's rank {decay_rank} at least 1")
+        self.proj, self.a2, self.o = Linear(), Linear(), Linear()        # proj: [W_a1; W_q; W_k; W_v; W_g] stacked
+        self.norm = None
+
+    @property
+    def q_col(self):
+        return self.rank
+
+    @property
+    def k_col(self):
+        return self.rank + self.H * self.hs
+
+    @property
+    def v_col(self):
+        return self.rank + 2 * self.H * self.hs
+
+    @property
+    def g_col(self):
+        return self.rank + 2 * self.H * self.hs + self.H * self.vd
+
+    def tensors(self):
+        D, A, B = self.hidden, self.H * self.hs, self.H * self.vd
+        return {"wq": ParamSpec((A, D)), "wk": ParamSpec((A, D)), "wv": ParamSpec((B, D)), "wg": ParamSpec((B, D)),
+                "wa1": ParamSpec((self.rank, D)), "wa2": ParamSpec((A, self.rank)), "a2_bias": ParamSpec((A,), "normal"),
+                "norm": ParamSpec((self.vd,), "ones"), "wo": ParamSpec((D, B))}
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wa1", "wq", "wk", "wv", "wg")], dim=0).contiguous()
+        self.proj.load(w, None, device, dtype)
+        self.a2.load(tensors["wa2"], tensors["a2_bias"], device, dtype)
+        self.o.load(tensors["wo"], None, device, dtype)
+        self.norm = upload(tensors["norm"], device, torch.float32).repeat(self.H).contiguous()      # the same for every head
+
+    def linears(self):
+        return [self.proj, self.o]
+
+    def cache_need(self) -> CacheNeed:
+        # per head a [head_dim, v_head_dim] matrix, float32, row-major
+        return CacheNeed(state=StateNeed((self.H * self.hs * self.vd,), torch.float32, device_addressed=True))
+
+    def forward(self, h, ctx, kv):
+        x = self.proj(h)
+        low = x[:, :self.rank]
+        if x.shape[0] > 1 and (x.stride(0) * x.element_size()) % 16:
+            low = low.contiguous()
+        z = self.a2(low, out_dtype=torch.float32)
+        o = ops.gla_scan(x, self.q_col, self.k_col, self.v_col, z, kv.state, ctx.slot_ids, self.H, self.hs, self.vd,
+                         self.hs ** -0.5, 1.0 / self.tau, **_sequences(ctx))
+        y = ops.head_norm_gate(o, x[:, self.g_col:], self.norm, self.H, self.vd, self.eps)
+        return self.o(y)
+
+
+@MIXERS.register("rglru")
+class RealGatedLRU(Part):
+    """A recurrent block around a real-gated linear recurrent unit, `width` channels wide (csrc/conv_scans.hip):
+        y = gelu_tanh(W_y h + b_y);   u = conv(W_x h + b_x)      a causal convolution per channel with a bias, no activation
+        r = sigmoid(A_b u_b + a_b),  i = sigmoid(I_b u_b + i_b)  u in `blocks` equal parts, a square matrix per part
+        log a = -sharpness r softplus(lam);  S <- a S + sqrt(1 - a^2) i u     from S = 0, the first token like any other
+        out = W_o (S * y)
+    The gates, a, the unit's operands and S are float32 (the gate matrices are kept in float32, turned to [in, out]); the
+    state row holds S, then the convolution's last taps - 1 inputs."""
+    prompt_capturable = True    # a prompt step is read from the context's device tensors alone
+
+    def __init__(self, hidden: int, width: int, blocks: int, conv_taps: int, sharpness: float = 8.0):
+        self.hidden, self.W, self.blocks, self.taps = int(hidden), int(width), int(blocks), int(conv_taps)
+        self.sharpness = float(sharpness)
+        if self.blocks < 1 or self.W % self.blocks:
+            raise ValueError(f"rglru: {width} channels are not {blocks} equal parts")
+        if not 1 <= self.taps <= ops.CONV_MAX_TAPS:
+            raise ValueError(f"rglru: conv_taps {conv_taps} (1 to {ops.CONV_MAX_TAPS})")
+        self.yx, self.o = Linear(), Linear()          # yx: [W_y; W_x] stacked with their biases
+        self.conv_w = self.conv_b = self.wa_t = self.wi_t = self.ba = self.bi = self.c_neg = None
+
+    def tensors(self):
+        D, W, B, bw = self.hidden, self.W, self.blocks, self.W // self.blocks
+        return {"wy": ParamSpec((W, D)), "by": ParamSpec((W,), "normal"), "wx": ParamSpec((W, D)), "bx": ParamSpec((W,), "normal"),
+                "conv": ParamSpec((W, self.taps)), "conv_bias": ParamSpec((W,), "normal"),
+                "ra": ParamSpec((B, bw, bw)), "ra_bias": ParamSpec((B, bw), "normal"),
+                "ri": ParamSpec((B, bw, bw)), "ri_bias": ParamSpec((B, bw), "normal"),
+                "lam": ParamSpec((W,), "normal"), "wo": ParamSpec((D, W))}
+
+    def load(self, tensors, device, dtype):
+        w = torch.cat([upload(tensors[n], device, dtype) for n in ("wy", "wx")], dim=0).contiguous()
+        b = torch.cat([upload(tensors[n], device, torch.float32) for n in ("by", "bx")])
+        self.yx.load(w, b, device, dtype)
+        self.o.load(tensors["wo"], None, device, dtype)
+        self.conv_w = upload(tensors["conv"], device, torch.float32)
+        self.conv_b = upload(tensors["conv_bias"], device, torch.float32)
+        self.wa_t = upload(tensors["ra"], device, torch.float32).transpose(1, 2).contiguous()
+        self.wi_t = upload(tensors["ri"], device, torch.float32).transpose(1, 2).contiguous()
+        self.ba = upload(tensors["ra_bias"], device, torch.float32).reshape(-1).contiguous()
+        self.bi = upload(tensors["ri_bias"], device, torch.float32).reshape(-1).contiguous()
+        lam = tensors["lam"].detach().to("cpu").to(torch.float64)
+        self.c_neg = (-self.sharpness * torch.nn.functional.softplus(lam)).to(torch.float32).to(device)
+
+    def linears(self):
+        return [self.yx, self.o]
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(state=StateNeed((self.W * self.taps,), torch.float32, device_addressed=True))
+
+    def forward(self, h, ctx, kv):
+        W = self.W
+        yx = self.yx(h)                                   # [T, 2 W]: the y branch before its gelu, then the convolution's input
+        seqs = _sequences(ctx)
+        conv_state = kv.state[:, W:] if self.taps > 1 else kv.state
+        u = ops.short_conv(yx, W, self.conv_w, self.conv_b, conv_state, ctx.positions, ctx.seq_index, ctx.slot_ids,
+                           out_dtype=torch.float32, **seqs)
+        a, b = ops.lru_gates(u, self.wa_t, self.ba, self.wi_t, self.bi, self.c_neg)
+        out = ops.lru_scan(a, b, yx[:, :W], kv.state, ctx.slot_ids, **seqs)
+        return self.o(out)
