@@ -141,9 +141,12 @@ def latent_attention(h, W, p, m, eps):
     q = (cq @ W[p + "uq"].T).reshape(T, H, d + r)
     dkv = h @ W[p + "dkv"].T
     c = unit_rms(dkv[:, :R], eps) * W[p + "dkv.norm"]
-    rot = dict(m["rot"], dims=r)
-    k_rot = rotate_halves(dkv[:, R:].reshape(T, 1, r), range(T), rot)[:, 0]
-    q_rot = rotate_halves(q[..., d:], range(T), rot)
+    if r:
+        rot = dict(m["rot"], dims=r)
+        k_rot = rotate_halves(dkv[:, R:].reshape(T, 1, r), range(T), rot)[:, 0]
+        q_rot = rotate_halves(q[..., d:], range(T), rot)
+    else:                                                 # no rotated part: the plain scores alone
+        k_rot, q_rot = torch.zeros((T, 0), dtype=F64), torch.zeros((T, H, 0), dtype=F64)
     k = (c @ W[p + "uk"].T).reshape(T, H, d)
     v = (c @ W[p + "uv"].T).reshape(T, H, vd)
     gate = sigmoid(h @ W[p + "g"].T)                      # [T, H]
@@ -218,14 +221,18 @@ def dense_unit(h, W, p, mlp):
     return (g * sigmoid(GATE_SLOPE * g) * (u + 1.0)) @ W[p + "down"].T
 
 
-def expert_mixture(h, W, p, mlp):
+def expert_mixture(h, W, p, mlp, margins=None):
     """Router logits W_router h + b; the `top` largest are chosen and weighted by the softmax over the chosen alone; an
-    expert is W_down (silu(W_gate h) * (W_up h))."""
+    expert is W_down (silu(W_gate h) * (W_up h)).  margins: a list of one number per token, lowered to the distance
+    between the last chosen logit and the first one left out."""
     z = h @ W[p + "router"].T + W[p + "router.b"]
     top = mlp["router"]["top"]
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         val, idx = torch.topk(z[t], top)
+        if margins is not None and top < z.shape[1]:
+            rest = torch.topk(z[t], top + 1)[0]
+            margins[t] = min(margins[t], float(rest[top - 1] - rest[top]))
         w = torch.softmax(val, dim=-1)
         for wt, e in zip(w.tolist(), idx.tolist()):
             q = f"{p}e{e}."
@@ -233,8 +240,8 @@ def expert_mixture(h, W, p, mlp):
     return out
 
 
-def feed_forward(h, W, p, mlp):
-    return dense_unit(h, W, p, mlp) if mlp["kind"] == "dense" else expert_mixture(h, W, p, mlp)
+def feed_forward(h, W, p, mlp, margins=None):
+    return dense_unit(h, W, p, mlp) if mlp["kind"] == "dense" else expert_mixture(h, W, p, mlp, margins)
 
 
 # ---- the model -------------------------------------------------------------------------------------------------
@@ -249,13 +256,16 @@ def layer_runs(cfg: dict):
     return list(range(a)) + list(range(a, b)) * loop["times"] + list(range(b, n))
 
 
-def forward(cfg: dict, W: dict, tokens, collect=None):
+def forward(cfg: dict, W: dict, tokens, collect=None, margins=None):
     """Logits [T, vocab] of one whole sequence.  collect: a list that receives the sum of the streams after every layer
     run.  The residual is `streams` copies of the embedding; a sublayer reads their sum weighted by `in`, and all copies
-    are rebuilt at once from the old ones: x_t <- sum_s mix[s, t] x_s + m out[t] y."""
+    are rebuilt at once from the old ones: x_t <- sum_s mix[s, t] x_s + m out[t] y.  Without `streams` in the configuration
+    there is one residual and x <- x + m y."""
     eps, m = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     S = cfg.get("streams")
     x0 = W["embed"][torch.as_tensor(list(tokens))]
+    if margins is not None:
+        margins[:] = [float("inf")] * len(tokens)          # margins: every token's smallest routing margin over the layers
     X = torch.stack([x0] * (S or 1))
 
     def sublayer(X, name, fn, q):
@@ -269,7 +279,7 @@ def forward(cfg: dict, W: dict, tokens, collect=None):
         L, p = cfg["layers"][i], f"l{i}."
         X = sublayer(X, p + "norm1", lambda hh: MIXERS[L["type"]](hh, W, p + "mix.", L["mixer"], eps), p + "hc1")
         if L.get("mlp") is not None:
-            X = sublayer(X, p + "norm2", lambda hh: feed_forward(hh, W, p + "mlp.", L["mlp"]), p + "hc2")
+            X = sublayer(X, p + "norm2", lambda hh: feed_forward(hh, W, p + "mlp.", L["mlp"], margins), p + "hc2")
         if collect is not None:
             collect.append(X.sum(0))
     return tanh_norm(X.sum(0), W, "final.norm") @ W["head"].T
