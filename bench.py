@@ -232,9 +232,40 @@ def _fazopel_configs(z):
     return (faz,) + _sonodra_configs(z)
 
 
+def _mutirax_configs(z):
+    """(Mutirax config.json, Fazopel config.json, Sonodra config.json, Llama config.json) of equal width, layer runs and
+    attention heads: a parallel layer (attention with a convolution on its projections beside a recurrent unit as wide as
+    the model), a gated-linear-attention layer and a latent-attention layer, repeated; three quarters of the layers are
+    stored and the first three run twice, so that as many layers run as the others have; four residual streams.  The
+    first layer's feed-forward is the dense unit, the others choose `top` of `experts` gated experts whose three matrices
+    are together as large as the gated feed-forward's."""
+    gated = _llama_config(z)["intermediate_size"]
+    moe = dict(kind="moe", expert=dict(ff=gated // z["top"] // 64 * 64), router=dict(experts=z["experts"], top=z["top"]))
+    H = z["heads"]
+    par = dict(left=dict(heads=H, kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], conv=4, scale=z["dim"] ** -0.5,
+                         rot=dict(base=500000.0, dims=z["rot_dims"])),
+               right=dict(width=z["right"], blocks=z["right"] // 256, conv=4))
+    gla = dict(heads=H, dim=z["dim"], vdim=z["dim"], tau=16.0, decay_rank=z["rank"])
+    lat = dict(heads=H, dim=z["dim"], rot_dim=z["rot_dims"], vdim=z["dim"], kv_rank=256 - z["rot_dims"], q_rank=z["width"] // 2,
+               scale=(z["dim"] + z["rot_dims"]) ** -0.5,
+               rot=dict(base=250000.0, dims=z["rot_dims"], scaling=dict(factor=8.0, original=1024, fast=32.0, slow=1.0)))
+    stored = z["layers"] - 3
+    layers = []
+    for i in range(stored):
+        mlp = dict(kind="dense", ff=gated, limit=7.0) if i == 0 else moe
+        kind, mixer = (("parallel", par), ("gla", gla), ("latent_attention", lat))[i % 3]
+        layers.append(dict(type=kind, mixer=mixer, mlp=mlp))
+    mut = dict(architecture="Mutirax", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-6), residual_mult=0.5, streams=4,
+               loop=dict(start=0, stop=3, times=2), layers=layers)
+    return (mut,) + _fazopel_configs(z)
+
+
 def _design_configs(design, z):
     """name -> config.json: the design, then what it is measured beside (the Llama-style decoder of equal width, layers,
-    attention heads and (nearly) equal weight bytes read per token; for Fazopel also Sonodra, the closest of the others)."""
+    attention heads and (nearly) equal weight bytes read per token; for Fazopel also Sonodra, the closest of the others;
+    for Mutirax Fazopel and Sonodra)."""
+    if design == "mutirax":
+        return dict(zip(("mutirax", "fazopel", "sonodra", "llama"), _mutirax_configs(z)))
     if design == "fazopel":
         return dict(zip(("fazopel", "sonodra", "llama"), _fazopel_configs(z)))
     if design == "sonodra":
@@ -348,7 +379,7 @@ def main() -> int:
     ap.add_argument("--prompt-lens", default=None, metavar="LO,HI", help="prompt lengths of the decode batches")
     ap.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="tokens of the measured prompt step")
     ap.add_argument("--design-alone", action="store_true", help="with --design: the design alone, for profiling")
-    ap.add_argument("--design", choices=["sunusun", "sonodra", "fazopel"], default=None,
+    ap.add_argument("--design", choices=["sunusun", "sonodra", "fazopel", "mutirax"], default=None,
                     help="instead of the benchmark: prefill and decode of this design beside the Llama-style decoder of equal "
                          "width, heads, layers and weight bytes, at the sizes of --design-size (random weights; one JSON line)")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="2048")

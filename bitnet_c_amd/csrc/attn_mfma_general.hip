@@ -393,8 +393,8 @@ __global__ __launch_bounds__(BN_WAVE) void attn_general_combine_kernel(bf16* __r
 
 static bool ag_size(int x, int unit) { return x == unit || x == 2 * unit || x == 3 * unit || x == 4 * unit || x == 8 * unit; }
 
-// 1 if the prompt kernel takes these head sizes (keys 32, 64, 96, 128 or 256 wide, values 32, 64, 96, 128 or 256)
-extern "C" int bn_attn_general_supports(int hs, int vd) { return (ag_size(hs, 32) && ag_size(vd, 32)) ? 1 : 0; }
+// 1 if the kernels take these head sizes (keys 32, 64, 96, 128 or 256 wide, values 32, 64, 96, 128, 192 or 256)
+extern "C" int bn_attn_general_supports(int hs, int vd) { return (ag_size(hs, 32) && (ag_size(vd, 32) || vd == 192)) ? 1 : 0; }
 
 template <int DC>
 static int ag_launch_dt(const GenArgs& a, int vd, dim3 grid, hipStream_t s) {
@@ -404,6 +404,7 @@ static int ag_launch_dt(const GenArgs& a, int vd, dim3 grid, hipStream_t s) {
         case 4: AG_CASE(4);
         case 6: AG_CASE(6);
         case 8: AG_CASE(8);
+        case 12: AG_CASE(12);
         case 16: AG_CASE(16);
     }
 #undef AG_CASE
@@ -442,6 +443,7 @@ static int ag_launch_decode_dt(const GenDecodeArgs& a, int vd, dim3 grid, hipStr
         case 4: AG_CASE(4);
         case 6: AG_CASE(6);
         case 8: AG_CASE(8);
+        case 12: AG_CASE(12);
         case 16: AG_CASE(16);
     }
 #undef AG_CASE

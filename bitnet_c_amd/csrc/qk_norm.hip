@@ -51,7 +51,9 @@ __device__ __forceinline__ void qkn_sincos(float a, float* sn, float* cs) {
 }
 
 // a workgroup takes QKN_WAVES heads of one row, a wave each; heads 0 .. H-1 are queries, then Hkv keys, then Hkv values.
-// With norms over the whole projections every workgroup of a row forms the two sums of squares for itself.
+// With norms over the whole projections one workgroup takes all heads of a row, its waves in turn: the query heads are
+// rewritten in place, so the sums of squares over the whole projections must have been formed (by all threads, in front
+// of a barrier) before any of them is, and no other workgroup may read the row meanwhile.
 template <typename T>
 __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNormArgs a) {
     __shared__ float scratch[16];
@@ -71,7 +73,9 @@ __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNo
         fk = 1.0f / sqrtf(sk / (float)nk + a.eps);
     }
     const int rd = a.inv_freq ? a.rope_dims : 0, half = rd / 2;
-    for (int head = blockIdx.y * QKN_WAVES + wave; head < min(a.H + 2 * a.Hkv, (int)(blockIdx.y + 1) * QKN_WAVES); head += QKN_WAVES) {
+    const int n_heads = a.H + 2 * a.Hkv;
+    const int head0 = a.norm_all ? 0 : blockIdx.y * QKN_WAVES, head1 = a.norm_all ? n_heads : min(n_heads, head0 + QKN_WAVES);
+    for (int head = head0 + wave; head < head1; head += QKN_WAVES) {
         const bool is_q = head < a.H, is_k = !is_q && head < a.H + a.Hkv;
         if (is_q || is_k) {
             if (is_k && !a.k_pages) continue;
@@ -155,7 +159,7 @@ extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positio
     a.eps = eps; a.temp_coef = temp_coef; a.temp_every = temp_every; a.v_transposed = v_transposed ? 1 : 0;
     a.norm_all = norm_all ? 1 : 0; a.rope_dims = inv_freq ? rope_dims : 0; a.rope_interleaved = rope_interleaved ? 1 : 0;
     a.v_from_k = v_from_k ? 1 : 0;
-    const dim3 grid(n_tokens, (H + 2 * Hkv + QKN_WAVES - 1) / QKN_WAVES), block(QKN_WAVES * BN_WAVE);
+    const dim3 grid(n_tokens, norm_all ? 1 : (H + 2 * Hkv + QKN_WAVES - 1) / QKN_WAVES), block(QKN_WAVES * BN_WAVE);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, 0, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, block, 0, s, a);
     else return BN_ERR_DTYPE;

@@ -1452,13 +1452,13 @@ def qk_norm_store(qkv: torch.Tensor, positions: torch.Tensor, H: int, Hkv: int, 
 GENERAL_PROMPT_TILE = 16       # query tokens of a tile of attention_general_prompt
 # BITNET_NO_GENERAL_MFMA=1 keeps the attention mixer's general form on the vector kernel in prompt steps too
 GENERAL_PROMPT_ON_MATRIX_CORES = os.environ.get("BITNET_NO_GENERAL_MFMA", "") in ("", "0")
-_GENERAL_SIZES = (32, 64, 96, 128, 256)
+_GENERAL_SIZES = (32, 64, 96, 128, 256)        # key widths; values may also be 192 wide (a latent beside a rotated key part)
 
 
 def attention_general_supported(dtype, hs: int, v_dim: int) -> bool:
     """Whether attention_general_prompt takes this type and these head sizes (bn_attn_general_supports, answered here so
     that asking loads no kernel)."""
-    return dtype == torch.bfloat16 and int(hs) in _GENERAL_SIZES and int(v_dim) in _GENERAL_SIZES
+    return dtype == torch.bfloat16 and int(hs) in _GENERAL_SIZES and int(v_dim) in _GENERAL_SIZES + (192,)
 
 
 def attention_general_prompt(qkv: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,

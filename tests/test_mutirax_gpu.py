@@ -457,6 +457,32 @@ def test_the_latent_and_its_rotated_part_in_the_pages(dtype, R, rot, scaled):
         assert torch.equal(got[..., :off].cpu(), heads[..., :off].to(dtype)) and torch.equal(qd[5].cpu(), q[5])
 
 
+@pytest.mark.parametrize("H,G,hs", [(6, 1, 8), (16, 4, 64), (5, 5, 34)])
+def test_a_norm_over_the_whole_projection_reads_it_before_any_head_is_rewritten(H, G, hs):
+    """The queries are rewritten in place, and the norm over the whole query projection needs all of them as they arrived:
+    with more heads than one workgroup's waves take at once, many rows, again and again, every result is the plain one; the
+    values are the keys as they arrived."""
+    from bitnet_c_amd import ops
+    from bitnet_c_amd.cache import PAGE
+    g = torch.Generator().manual_seed(H + hs)
+    T, eps = 128, 1e-5
+    qk = torch.randn(T, (H + G) * hs, generator=g)
+    wq, wk = 1 + 0.2 * torch.randn(H * hs, generator=g), 1 + 0.2 * torch.randn(G * hs, generator=g)
+    rot = dict(base=100.0, dims=hs // 2 * 2)
+    from bitnet_c_amd.parts.position import rope_frequencies
+    inv = rope_frequencies(rot["dims"], rot["base"]).to(DEV)
+    q = pm.rotate_halves((pm.unit_rms(qk[:, :H * hs].double(), eps) * wq.double()).view(T, H, hs), range(T), rot)
+    kp = torch.zeros(2, G, PAGE, hs, device=DEV)
+    vp = torch.zeros(2, G, hs, PAGE, device=DEV)
+    for _ in range(30):
+        x = qk.to(DEV).clone()
+        ops.qk_norm_store(x, i32(list(range(T))), H, G, hs, q_weight=f32(wq), k_weight=f32(wk), eps=eps, seq_index=i32([0] * T),
+                          block_table=i32([[1, 0]]), k_pages=kp, v_pages=vp, v_transposed=True, inv_freq=inv, rope_dims=rot["dims"],
+                          norm_projection=True, v_from_k=True)
+        assert rel_err(x[:, :H * hs], q.reshape(T, -1)) < 2e-4
+        assert torch.equal(vp[0, :, :, 5].cpu(), qk[PAGE + 5, H * hs:].view(G, hs))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T", [1, 5, 40])
 def test_a_product_per_head_with_one_gate_number_per_head(dtype, T):
@@ -668,6 +694,22 @@ def test_the_convolution_sees_exactly_its_taps(tmp_path, dtype):
         parts.append(eng.step([bn.StepEntry(s, toks[at:at + p], list(range(p)))]))
         at += p
     close(torch.cat(parts), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_wide_latent_beside_its_rotated_part(tmp_path, dtype):
+    """A latent of 192 numbers beside 64 rotated ones: key rows of 256, values of 192, the widths at which the prompt and
+    decode steps of the latent mixer run on the matrix cores in bfloat16.  A prompt across a page's border, then decoded."""
+    import bitnet_c_amd as bn
+    cfg = _model(59, 64, 1e-5, 0.5, [_lat(3, 16, 64, 24, 192, 40, 0.11, (250000.0, 8.0, 1024, 32.0, 1.0), None)], streams=2)
+    folder = write_folder(tmp_path / "wide", cfg, 6)
+    toks = torch.randint(0, 59, (90,), generator=torch.Generator().manual_seed(4)).tolist()
+    want = plain(folder, toks)
+    eng = engine(folder, dtype)
+    s = eng.new_sequence()
+    got = eng.step([bn.StepEntry(s, toks[:70], list(range(70)))])
+    dec = torch.cat([eng.step([bn.StepEntry(s, [t], [0])]) for t in toks[70:]])
+    close(torch.cat([got, dec]), want, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
