@@ -8,7 +8,7 @@
 //                   channel; the unit's two operands a and sqrt(1 - a^2) i u leave as float32 rows
 //   bn_lru_scan     S <- a S + b per channel, the result times gelu_tanh of the other branch
 //   bn_gla_scan     gated linear attention: per head S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T q_t with a decay per key
-//                   channel and token, alpha = sigmoid(z)^(1 / tau)
+//                   channel and token, alpha = sigmoid(z)^(1 / tau); token by token, the tokens staged two runs deep
 //
 // Everything that enters a recurrence is float32: gates, decays and their logarithms, exponentials, the state.  Every
 // chain is the same operations in the same order whatever else a step holds, so a sequence's values do not depend on
@@ -284,61 +284,93 @@ struct GlaArgs {
     float q_scale, inv_tau;
 };
 
-// A wave owns (sequence, head, 16 value columns).  Lane = (slice s of the key channels, column c): it keeps rows
-// s, s + 4, s + 8, ... of its column of S in registers.  Tokens come in runs of 16: the wave stages q (scaled), k and
-// alpha of the run as float32 in shared memory (alpha = exp(logsigmoid(z) / tau)), then walks the run; the four slices'
-// parts of o meet through two lane exchanges in a fixed order.
-template <typename T, int RPL>
-__global__ __launch_bounds__(BN_WAVE) void gla_scan_kernel(GlaArgs a) {
+// A wave owns (sequence, head, 16 value columns); a workgroup is NW such waves over neighbouring columns of one head, so
+// that q, k and the decays of a token are staged once for 16 NW columns.  Lane = (slice s of the key channels, column c):
+// it keeps rows s, s + 4, s + 8, ... of its column of S in registers.  Tokens come in runs of GLA_RUN: all threads turn a
+// run into q (scaled), k, alpha = exp(logsigmoid(z) / tau) and v as float32 in shared memory, in two buffers: the next
+// run's loads are asked for before the current run is walked and parked behind it, so the chain waits for no memory.
+// The four slices' parts of o meet through two lane exchanges in a fixed order; the chain of a column is the same
+// operations in the same order whatever the step holds and however many waves share the workgroup.
+template <typename T, int RPL, int NW>
+__global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
     constexpr int DKP = GLA_SLICES * RPL;                 // staged key channels (those past dk are zeros)
-    __shared__ float q_s[GLA_RUN][DKP], k_s[GLA_RUN][DKP], a_s[GLA_RUN][DKP], v_s[GLA_RUN][GLA_COLS];
+    constexpr int RUN = RPL == 64 ? 8 : GLA_RUN;          // tokens of a run (fewer for the widest heads: shared memory)
+    constexpr int NT = BN_WAVE * NW, VC = GLA_COLS * NW;
+    constexpr int PF = (RUN * DKP + NT - 1) / NT, PV = (RUN * VC + NT - 1) / NT;
+    __shared__ float q_s[2][RUN][DKP], k_s[2][RUN][DKP], a_s[2][RUN][DKP], v_s[2][RUN][VC];
     const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
     if (sr.n <= 0 || sr.pos0 < 0) return;
-    const int head = blockIdx.y, col0 = blockIdx.z * GLA_COLS;
-    const int lane = threadIdx.x, sl = lane >> 4, c = lane & 15;
-    const bool has = col0 + c < a.dv;
+    const int head = blockIdx.y, colb = blockIdx.z * VC;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, sl = lane >> 4, c = lane & 15;
+    const int col = colb + wave * GLA_COLS + c;
+    const bool has = col < a.dv;
     const T* x = reinterpret_cast<const T*>(a.x);
-    float* sp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * a.dk * a.dv + col0 + c;
+    float* sp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * a.dk * a.dv + (has ? col : 0);
     float S[RPL];
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
         const int i = sl + GLA_SLICES * r;
         S[r] = (sr.pos0 > 0 && has && i < a.dk) ? sp[(size_t)i * a.dv] : 0.f;
     }
-    for (int t0 = 0; t0 < sr.n; t0 += GLA_RUN) {
-        const int run = min(GLA_RUN, sr.n - t0);
-        __syncthreads();
-        for (int idx = lane; idx < GLA_RUN * DKP; idx += BN_WAVE) {
-            const int tt = idx / DKP, i = idx - tt * DKP;
-            float qv = 0.f, kv = 0.f, al = 0.f;
-            if (tt < run && i < a.dk) {
-                const size_t row = (size_t)(sr.row0 + t0 + tt);
-                qv = to_f32(x[row * a.ld + a.q_col + head * a.dk + i]) * a.q_scale;
-                kv = to_f32(x[row * a.ld + a.k_col + head * a.dk + i]);
-                const float zz = a.z[row * (size_t)(a.H * a.dk) + (size_t)head * a.dk + i];
-                al = expf((fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * a.inv_tau);
-            }
-            q_s[tt][i] = qv; k_s[tt][i] = kv; a_s[tt][i] = al;
+    float rq[PF], rk[PF], rz[PF], rv[PV];
+    // loads from clamped places, unconditional: what lies outside the run or the head is never parked
+    auto fetch = [&](int t0) {
+        const int run = min(RUN, sr.n - t0);
+#pragma unroll
+        for (int k = 0; k < PF; ++k) {
+            const int e = tid + k * NT, tt = min(e / DKP, run - 1), i = min(e % DKP, a.dk - 1);
+            const size_t row = (size_t)(sr.row0 + t0 + tt);
+            rq[k] = to_f32(x[row * a.ld + a.q_col + head * a.dk + i]);
+            rk[k] = to_f32(x[row * a.ld + a.k_col + head * a.dk + i]);
+            rz[k] = a.z[row * (size_t)(a.H * a.dk) + (size_t)head * a.dk + i];
         }
-        for (int idx = lane; idx < GLA_RUN * GLA_COLS; idx += BN_WAVE) {
-            const int tt = idx / GLA_COLS, cc = idx - tt * GLA_COLS;
-            v_s[tt][cc] = (tt < run && col0 + cc < a.dv)
-                              ? to_f32(x[(size_t)(sr.row0 + t0 + tt) * a.ld + a.v_col + head * a.dv + col0 + cc]) : 0.f;
+#pragma unroll
+        for (int k = 0; k < PV; ++k) {
+            const int e = tid + k * NT, tt = min(e / VC, run - 1), cc = min(colb + e % VC, a.dv - 1);
+            rv[k] = to_f32(x[(size_t)(sr.row0 + t0 + tt) * a.ld + a.v_col + head * a.dv + cc]);
         }
-        __syncthreads();
+    };
+    auto park = [&](int buf, int t0) {
+        const int run = min(RUN, sr.n - t0);
+#pragma unroll
+        for (int k = 0; k < PF; ++k) {
+            const int e = tid + k * NT, tt = e / DKP, i = e % DKP;
+            if (e >= RUN * DKP) break;
+            const bool ok = tt < run && i < a.dk;
+            q_s[buf][tt][i] = ok ? rq[k] * a.q_scale : 0.f;
+            k_s[buf][tt][i] = ok ? rk[k] : 0.f;
+            a_s[buf][tt][i] = ok ? expf((fminf(rz[k], 0.f) - log1pf(expf(-fabsf(rz[k])))) * a.inv_tau) : 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < PV; ++k) {
+            const int e = tid + k * NT, tt = e / VC, cc = e % VC;
+            if (e >= RUN * VC) break;
+            v_s[buf][tt][cc] = (tt < run && colb + cc < a.dv) ? rv[k] : 0.f;
+        }
+    };
+    fetch(0);
+    park(0, 0);
+    __syncthreads();
+    int buf = 0;
+    for (int t0 = 0; t0 < sr.n; t0 += RUN, buf ^= 1) {
+        const int run = min(RUN, sr.n - t0);
+        const bool more = t0 + RUN < sr.n;
+        if (more) fetch(t0 + RUN);
         for (int tt = 0; tt < run; ++tt) {
-            const float vj = v_s[tt][c];
+            const float vj = v_s[buf][tt][wave * GLA_COLS + c];
             float o = 0.f;
 #pragma unroll
             for (int r = 0; r < RPL; ++r) {
                 const int i = sl + GLA_SLICES * r;
-                S[r] = fmaf(a_s[tt][i], S[r], k_s[tt][i] * vj);
-                o = fmaf(S[r], q_s[tt][i], o);
+                S[r] = fmaf(a_s[buf][tt][i], S[r], k_s[buf][tt][i] * vj);
+                o = fmaf(S[r], q_s[buf][tt][i], o);
             }
             o += __shfl_xor(o, 16, BN_WAVE);
             o += __shfl_xor(o, 32, BN_WAVE);
-            if (sl == 0 && has) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col0 + c] = o;
+            if (sl == 0 && has) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col] = o;
         }
+        if (more) park(buf ^ 1, t0 + RUN);
+        __syncthreads();
     }
     if (has) {
 #pragma unroll
@@ -351,14 +383,27 @@ __global__ __launch_bounds__(BN_WAVE) void gla_scan_kernel(GlaArgs a) {
 
 extern "C" int bn_gla_supports(int dk, int dv) { return (dk >= 1 && dk <= GLA_MAX_DIM && dv >= 1) ? 1 : 0; }
 
-template <typename T>
-static int gla_launch(const GlaArgs& a, dim3 grid, hipStream_t s) {
+// waves of a workgroup: as many as cover a head's value columns, up to eight
+static int gla_waves(int dv) { return dv <= GLA_COLS ? 1 : dv <= 4 * GLA_COLS ? 4 : 8; }
+
+template <typename T, int NW>
+static int gla_launch_nw(const GlaArgs& a, int n_seqs, hipStream_t s) {
+    const dim3 grid(n_seqs, a.H, (a.dv + GLA_COLS * NW - 1) / (GLA_COLS * NW)), block(BN_WAVE * NW);
     const int rpl = (a.dk + GLA_SLICES - 1) / GLA_SLICES;
-    if (rpl <= 8) hipLaunchKernelGGL((gla_scan_kernel<T, 8>), grid, dim3(BN_WAVE), 0, s, a);
-    else if (rpl <= 16) hipLaunchKernelGGL((gla_scan_kernel<T, 16>), grid, dim3(BN_WAVE), 0, s, a);
-    else if (rpl <= 32) hipLaunchKernelGGL((gla_scan_kernel<T, 32>), grid, dim3(BN_WAVE), 0, s, a);
-    else hipLaunchKernelGGL((gla_scan_kernel<T, 64>), grid, dim3(BN_WAVE), 0, s, a);
+    if (rpl <= 8) hipLaunchKernelGGL((gla_scan_kernel<T, 8, NW>), grid, block, 0, s, a);
+    else if (rpl <= 16) hipLaunchKernelGGL((gla_scan_kernel<T, 16, NW>), grid, block, 0, s, a);
+    else if (rpl <= 32) hipLaunchKernelGGL((gla_scan_kernel<T, 32, NW>), grid, block, 0, s, a);
+    else hipLaunchKernelGGL((gla_scan_kernel<T, 64, NW>), grid, block, 0, s, a);
     return bn_launch_status();
+}
+
+template <typename T>
+static int gla_launch(const GlaArgs& a, int n_seqs, hipStream_t s) {
+    switch (gla_waves(a.dv)) {
+        case 1: return gla_launch_nw<T, 1>(a, n_seqs, s);
+        case 4: return gla_launch_nw<T, 4>(a, n_seqs, s);
+        default: return gla_launch_nw<T, 8>(a, n_seqs, s);
+    }
 }
 
 extern "C" int bn_gla_scan(int dtype, const void* x, int ld, int q_col, int k_col, int v_col, const float* z, float* o,
@@ -371,8 +416,7 @@ extern "C" int bn_gla_scan(int dtype, const void* x, int ld, int q_col, int k_co
     a.x = x; a.z = z; a.o = o; a.state = state; a.tiles = tiles; a.seq_lens = seq_lens; a.slot_ids = slot_ids;
     a.state_stride = state_stride; a.ld = ld; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col; a.H = H; a.dk = dk; a.dv = dv;
     a.q_scale = q_scale; a.inv_tau = inv_tau;
-    const dim3 grid(n_seqs, H, (dv + GLA_COLS - 1) / GLA_COLS);
-    if (dtype == BN_DT_F32) return gla_launch<float>(a, grid, s);
-    if (dtype == BN_DT_BF16) return gla_launch<bf16>(a, grid, s);
+    if (dtype == BN_DT_F32) return gla_launch<float>(a, n_seqs, s);
+    if (dtype == BN_DT_BF16) return gla_launch<bf16>(a, n_seqs, s);
     return BN_ERR_DTYPE;
 }
