@@ -20,7 +20,6 @@
 #define GLA_MAX_DIM 256           // key channels of a head (the Python side reads this line)
 #define GLA_COLS 16               // value columns of a wave
 #define GLA_SLICES 4              // parts of the key channels, 16 lanes each
-#define GLA_RUN 16                // tokens staged at once
 
 struct SeqRange { int seq, row0, n, pos0; };
 
@@ -157,47 +156,66 @@ extern "C" int bn_short_conv(int in_dtype, int out_dtype, const void* x, int ldx
 
 // ---- gates of the real-gated linear recurrent unit ----------------------------------------------------------------
 #define LRU_ROWS 8
-#define LRU_COLS 128
+#define LRU_COLS 64
+#define LRU_SLICES 8
 
-// One workgroup a (eight rows, block of the input, 128 output channels of the block).  The rows' part of u is staged in
-// shared memory; a thread owns an output channel and walks the part's inputs in order with both matrices, which lie
-// [block][in][out] so that the threads of a wave read neighbouring words.
-__global__ __launch_bounds__(LRU_COLS) void lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ wa,
-                                                             const float* __restrict__ ba, const float* __restrict__ wi,
-                                                             const float* __restrict__ bi, const float* __restrict__ c_neg,
-                                                             float* __restrict__ a_out, float* __restrict__ b_out, int T,
-                                                             int W, int bw) {
-    extern __shared__ float us[];                        // [LRU_ROWS][bw]
-    const int t0 = blockIdx.x * LRU_ROWS, blk = blockIdx.y, o = blockIdx.z * LRU_COLS + threadIdx.x;
+// One workgroup a (eight rows, block of the input, 64 output channels of the block).  The rows' part of u is staged in
+// shared memory; a thread owns an output channel and one of eight runs of the part's inputs, which it walks in order with
+// both matrices (they lie [block][in][out], so the threads of a wave read neighbouring words); the runs' sums meet in
+// shared memory and are added in run order.  The sums of a row are the same operations whatever the step holds.
+__global__ __launch_bounds__(LRU_COLS * LRU_SLICES) void lru_gates_kernel(const float* __restrict__ u, const float* __restrict__ wa,
+                                                                          const float* __restrict__ ba, const float* __restrict__ wi,
+                                                                          const float* __restrict__ bi, const float* __restrict__ c_neg,
+                                                                          float* __restrict__ a_out, float* __restrict__ b_out, int T,
+                                                                          int W, int bw) {
+    extern __shared__ float us[];                        // [LRU_ROWS][bw], then the runs' sums [LRU_SLICES][LRU_ROWS][2][LRU_COLS]
+    float* red = us + LRU_ROWS * bw;
+    const int t0 = blockIdx.x * LRU_ROWS, blk = blockIdx.y, c = threadIdx.x & (LRU_COLS - 1), slice = threadIdx.x / LRU_COLS;
+    const int o = blockIdx.z * LRU_COLS + c;
     const int rows = min(LRU_ROWS, T - t0);
-    for (int idx = threadIdx.x; idx < LRU_ROWS * bw; idx += LRU_COLS) {
+    for (int idx = threadIdx.x; idx < LRU_ROWS * bw; idx += LRU_COLS * LRU_SLICES) {
         const int r = idx / bw, i = idx - r * bw;
         us[idx] = r < rows ? u[(size_t)(t0 + r) * W + (size_t)blk * bw + i] : 0.f;
     }
     __syncthreads();
-    if (o >= bw) return;
     float acc_a[LRU_ROWS], acc_i[LRU_ROWS];
 #pragma unroll
     for (int r = 0; r < LRU_ROWS; ++r) { acc_a[r] = 0.f; acc_i[r] = 0.f; }
-    const float* pa = wa + (size_t)blk * bw * bw + o;
-    const float* pi = wi + (size_t)blk * bw * bw + o;
-#pragma unroll 4
-    for (int i = 0; i < bw; ++i) {
-        const float va = pa[(size_t)i * bw], vi = pi[(size_t)i * bw];
+    const int per = (bw + LRU_SLICES - 1) / LRU_SLICES, i0 = slice * per, i1 = min(bw, i0 + per);
+    if (o < bw) {
+        const float* pa = wa + (size_t)blk * bw * bw + o;
+        const float* pi = wi + (size_t)blk * bw * bw + o;
+#pragma unroll 8
+        for (int i = i0; i < i1; ++i) {
+            const float va = pa[(size_t)i * bw], vi = pi[(size_t)i * bw];
 #pragma unroll
-        for (int r = 0; r < LRU_ROWS; ++r) {
-            const float x = us[r * bw + i];
-            acc_a[r] = fmaf(va, x, acc_a[r]);
-            acc_i[r] = fmaf(vi, x, acc_i[r]);
+            for (int r = 0; r < LRU_ROWS; ++r) {
+                const float x = us[r * bw + i];
+                acc_a[r] = fmaf(va, x, acc_a[r]);
+                acc_i[r] = fmaf(vi, x, acc_i[r]);
+            }
         }
     }
+#pragma unroll
+    for (int r = 0; r < LRU_ROWS; ++r) {
+        red[((slice * LRU_ROWS + r) * 2 + 0) * LRU_COLS + c] = acc_a[r];
+        red[((slice * LRU_ROWS + r) * 2 + 1) * LRU_COLS + c] = acc_i[r];
+    }
+    __syncthreads();
+    if (slice != 0 || o >= bw) return;
     const int ch = blk * bw + o;
     const float biasa = ba[ch], biasi = bi[ch], cn = c_neg[ch];
 #pragma unroll
     for (int r = 0; r < LRU_ROWS; ++r) {
         if (r >= rows) break;
-        const float rg = 1.0f / (1.0f + expf(-(acc_a[r] + biasa)));
-        const float ig = 1.0f / (1.0f + expf(-(acc_i[r] + biasi)));
+        float sa = 0.f, si = 0.f;
+#pragma unroll
+        for (int k = 0; k < LRU_SLICES; ++k) {
+            sa += red[((k * LRU_ROWS + r) * 2 + 0) * LRU_COLS + c];
+            si += red[((k * LRU_ROWS + r) * 2 + 1) * LRU_COLS + c];
+        }
+        const float rg = 1.0f / (1.0f + expf(-(sa + biasa)));
+        const float ig = 1.0f / (1.0f + expf(-(si + biasi)));
         const float la = cn * rg;                                  // log a <= 0
         const float m = sqrtf(fmaxf(-expm1f(2.0f * la), 0.f));      // sqrt(1 - a^2) without the cancellation near a = 1
         a_out[(size_t)(t0 + r) * W + ch] = expf(la);
@@ -209,11 +227,11 @@ extern "C" int bn_lru_gates(const float* u, const float* wa, const float* ba, co
                             const float* c_neg, float* a_out, float* b_out, int T, int W, int blocks, hipStream_t s) {
     if (T <= 0 || W <= 0 || blocks <= 0 || W % blocks || !u || !wa || !ba || !wi || !bi || !c_neg || !a_out || !b_out) return BN_ERR_ARG;
     const int bw = W / blocks;
-    const size_t shm = (size_t)LRU_ROWS * bw * sizeof(float);
+    const size_t shm = ((size_t)LRU_ROWS * bw + (size_t)LRU_SLICES * LRU_ROWS * 2 * LRU_COLS) * sizeof(float);
     const int row_tiles = (T + LRU_ROWS - 1) / LRU_ROWS;
     if (shm > 64 * 1024 || blocks > 65535 || (bw + LRU_COLS - 1) / LRU_COLS > 65535) return BN_ERR_ARG;
     const dim3 grid(row_tiles, blocks, (bw + LRU_COLS - 1) / LRU_COLS);
-    hipLaunchKernelGGL(lru_gates_kernel, grid, dim3(LRU_COLS), shm, s, u, wa, ba, wi, bi, c_neg, a_out, b_out, T, W, bw);
+    hipLaunchKernelGGL(lru_gates_kernel, grid, dim3(LRU_COLS * LRU_SLICES), shm, s, u, wa, ba, wi, bi, c_neg, a_out, b_out, T, W, bw);
     return bn_launch_status();
 }
 
@@ -286,7 +304,9 @@ struct GlaArgs {
 
 // A wave owns (sequence, head, 16 value columns); a workgroup is NW such waves over neighbouring columns of one head, so
 // that q, k and the decays of a token are staged once for 16 NW columns.  Lane = (slice s of the key channels, column c):
-// it keeps rows s, s + 4, s + 8, ... of its column of S in registers.  Tokens come in runs of GLA_RUN: all threads turn a
+// it keeps rows s RPL .. s RPL + RPL - 1 of its column of S in registers and reads their q, k and decays from shared memory
+// four at a time (a slice's run of a staged row is padded so that the four slices' reads fall into different banks).
+// Tokens come in runs: all threads turn a
 // run into q (scaled), k, alpha = exp(logsigmoid(z) / tau) and v as float32 in shared memory, in two buffers: the next
 // run's loads are asked for before the current run is walked and parked behind it, so the chain waits for no memory.
 // The four slices' parts of o meet through two lane exchanges in a fixed order; the chain of a column is the same
@@ -294,10 +314,12 @@ struct GlaArgs {
 template <typename T, int RPL, int NW>
 __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
     constexpr int DKP = GLA_SLICES * RPL;                 // staged key channels (those past dk are zeros)
-    constexpr int RUN = RPL == 64 ? 8 : GLA_RUN;          // tokens of a run (fewer for the widest heads: shared memory)
+    constexpr int SLP = RPL + 4, DKL = GLA_SLICES * SLP;  // a slice's channels and four floats of padding; a staged row
+    constexpr int RUN = 4;                                // tokens of a run
     constexpr int NT = BN_WAVE * NW, VC = GLA_COLS * NW;
     constexpr int PF = (RUN * DKP + NT - 1) / NT, PV = (RUN * VC + NT - 1) / NT;
-    __shared__ float q_s[2][RUN][DKP], k_s[2][RUN][DKP], a_s[2][RUN][DKP], v_s[2][RUN][VC];
+    __shared__ __align__(16) float q_s[2][RUN][DKL], k_s[2][RUN][DKL], a_s[2][RUN][DKL];
+    __shared__ float v_s[2][RUN][VC];
     const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
     if (sr.n <= 0 || sr.pos0 < 0) return;
     const int head = blockIdx.y, colb = blockIdx.z * VC;
@@ -309,7 +331,7 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
     float S[RPL];
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
-        const int i = sl + GLA_SLICES * r;
+        const int i = sl * RPL + r;
         S[r] = (sr.pos0 > 0 && has && i < a.dk) ? sp[(size_t)i * a.dv] : 0.f;
     }
     float rq[PF], rk[PF], rz[PF], rv[PV];
@@ -337,9 +359,10 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
             const int e = tid + k * NT, tt = e / DKP, i = e % DKP;
             if (e >= RUN * DKP) break;
             const bool ok = tt < run && i < a.dk;
-            q_s[buf][tt][i] = ok ? rq[k] * a.q_scale : 0.f;
-            k_s[buf][tt][i] = ok ? rk[k] : 0.f;
-            a_s[buf][tt][i] = ok ? expf((fminf(rz[k], 0.f) - log1pf(expf(-fabsf(rz[k])))) * a.inv_tau) : 0.f;
+            const int at = (i / RPL) * SLP + i % RPL;
+            q_s[buf][tt][at] = ok ? rq[k] * a.q_scale : 0.f;
+            k_s[buf][tt][at] = ok ? rk[k] : 0.f;
+            a_s[buf][tt][at] = ok ? expf((fminf(rz[k], 0.f) - log1pf(expf(-fabsf(rz[k])))) * a.inv_tau) : 1.0f;
         }
 #pragma unroll
         for (int k = 0; k < PV; ++k) {
@@ -356,18 +379,41 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
         const int run = min(RUN, sr.n - t0);
         const bool more = t0 + RUN < sr.n;
         if (more) fetch(t0 + RUN);
-        for (int tt = 0; tt < run; ++tt) {
-            const float vj = v_s[buf][tt][wave * GLA_COLS + c];
-            float o = 0.f;
+        // Rows outside, tokens inside: four rows of S walk the run's tokens while the next four rows' q, k and decays are
+        // on their way from shared memory, and the slices' parts of the run's outputs meet once, behind the run.  A place
+        // of the run without a token is staged as the identity (decay 1, k = q = v = 0): S passes it unchanged.
+        float vj[RUN], o[RUN];
 #pragma unroll
-            for (int r = 0; r < RPL; ++r) {
-                const int i = sl + GLA_SLICES * r;
-                S[r] = fmaf(a_s[buf][tt][i], S[r], k_s[buf][tt][i] * vj);
-                o = fmaf(S[r], q_s[buf][tt][i], o);
+        for (int tt = 0; tt < RUN; ++tt) { vj[tt] = v_s[buf][tt][wave * GLA_COLS + c]; o[tt] = 0.f; }
+        float4 av[2][RUN], kv[2][RUN], qv[2][RUN];
+        auto rows4 = [&](int set, int r) {
+#pragma unroll
+            for (int tt = 0; tt < RUN; ++tt) {
+                av[set][tt] = *reinterpret_cast<const float4*>(&a_s[buf][tt][sl * SLP + r]);
+                kv[set][tt] = *reinterpret_cast<const float4*>(&k_s[buf][tt][sl * SLP + r]);
+                qv[set][tt] = *reinterpret_cast<const float4*>(&q_s[buf][tt][sl * SLP + r]);
             }
-            o += __shfl_xor(o, 16, BN_WAVE);
-            o += __shfl_xor(o, 32, BN_WAVE);
-            if (sl == 0 && has) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col] = o;
+        };
+        rows4(0, 0);
+#pragma unroll
+        for (int r = 0; r < RPL; r += 4) {
+            const int set = (r / 4) & 1;
+            if (r + 4 < RPL) rows4(set ^ 1, r + 4);             // asked for before this group's rows are walked
+#pragma unroll
+            for (int tt = 0; tt < RUN; ++tt) {
+                S[r] = fmaf(av[set][tt].x, S[r], kv[set][tt].x * vj[tt]);         o[tt] = fmaf(S[r], qv[set][tt].x, o[tt]);
+                S[r + 1] = fmaf(av[set][tt].y, S[r + 1], kv[set][tt].y * vj[tt]); o[tt] = fmaf(S[r + 1], qv[set][tt].y, o[tt]);
+                S[r + 2] = fmaf(av[set][tt].z, S[r + 2], kv[set][tt].z * vj[tt]); o[tt] = fmaf(S[r + 2], qv[set][tt].z, o[tt]);
+                S[r + 3] = fmaf(av[set][tt].w, S[r + 3], kv[set][tt].w * vj[tt]); o[tt] = fmaf(S[r + 3], qv[set][tt].w, o[tt]);
+            }
+            __builtin_amdgcn_sched_barrier(0);                   // the compiler keeps to one group ahead (registers)
+        }
+#pragma unroll
+        for (int tt = 0; tt < RUN; ++tt) {
+            float v = o[tt];
+            v += __shfl_xor(v, 16, BN_WAVE);
+            v += __shfl_xor(v, 32, BN_WAVE);
+            if (tt < run && sl == 0 && has) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col] = v;
         }
         if (more) park(buf ^ 1, t0 + RUN);
         __syncthreads();
@@ -375,7 +421,7 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
     if (has) {
 #pragma unroll
         for (int r = 0; r < RPL; ++r) {
-            const int i = sl + GLA_SLICES * r;
+            const int i = sl * RPL + r;
             if (i < a.dk) sp[(size_t)i * a.dv] = S[r];
         }
     }
@@ -383,8 +429,9 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
 
 extern "C" int bn_gla_supports(int dk, int dv) { return (dk >= 1 && dk <= GLA_MAX_DIM && dv >= 1) ? 1 : 0; }
 
-// waves of a workgroup: as many as cover a head's value columns, up to eight
-static int gla_waves(int dv) { return dv <= GLA_COLS ? 1 : dv <= 4 * GLA_COLS ? 4 : 8; }
+// waves of a workgroup: four (64 value columns share a staged run) unless a head has no more than one wave's columns;
+// more waves a workgroup would share the staging further but put several chains on one SIMD
+static int gla_waves(int dv) { return dv <= GLA_COLS ? 1 : 4; }
 
 template <typename T, int NW>
 static int gla_launch_nw(const GlaArgs& a, int n_seqs, hipStream_t s) {
@@ -401,8 +448,7 @@ template <typename T>
 static int gla_launch(const GlaArgs& a, int n_seqs, hipStream_t s) {
     switch (gla_waves(a.dv)) {
         case 1: return gla_launch_nw<T, 1>(a, n_seqs, s);
-        case 4: return gla_launch_nw<T, 4>(a, n_seqs, s);
-        default: return gla_launch_nw<T, 8>(a, n_seqs, s);
+        default: return gla_launch_nw<T, 4>(a, n_seqs, s);
     }
 }
 

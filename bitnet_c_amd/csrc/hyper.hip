@@ -38,54 +38,58 @@ struct HcArgs {
     float mult;
 };
 
+// One thread a (row, column); the coefficients wait in shared memory.
 template <typename TD, typename TH>
 __global__ __launch_bounds__(256) void hc_step_kernel(HcArgs a) {
-    const int r = blockIdx.x;
+    __shared__ float cm[BN_HC_MAX_STREAMS * BN_HC_MAX_STREAMS], co[BN_HC_MAX_STREAMS], ci[BN_HC_MAX_STREAMS];
+    const int n = a.n;
+    if (threadIdx.x < n * n) cm[threadIdx.x] = a.delta ? a.mix[threadIdx.x] : 0.f;
+    if (threadIdx.x < n) {
+        co[threadIdx.x] = a.delta ? a.outc[threadIdx.x] : 0.f;
+        ci[threadIdx.x] = a.inc ? a.inc[threadIdx.x] : 1.0f;
+    }
+    __syncthreads();
+    const int r = blockIdx.x, d = blockIdx.y * blockDim.x + threadIdx.x;
     const int t = a.rows ? a.rows[r] : r;
-    if (t < 0 || t >= a.T) return;
+    if (t < 0 || t >= a.T || d >= a.D) return;
     const TD* delta = reinterpret_cast<const TD*>(a.delta);
     TH* h = reinterpret_cast<TH*>(a.h);
-    const float alpha = a.w ? a.alpha[0] : 0.f;
-    const int n = a.n;
-    for (int d = threadIdx.x; d < a.D; d += blockDim.x) {
-        const size_t at = (size_t)t * a.D + d;
-        float x[BN_HC_MAX_STREAMS];
+    const size_t at = (size_t)t * a.D + d;
+    float x[BN_HC_MAX_STREAMS];
 #pragma unroll
-        for (int s = 0; s < BN_HC_MAX_STREAMS; ++s) x[s] = s < n ? a.lanes_in[(size_t)s * a.in_stride + at] : 0.f;
-        if (delta) {
-            float y = 0.f;
-            for (int p = 0; p < a.n_slabs; ++p) y += to_f32(delta[(size_t)p * a.slab_stride + at]);
-            y *= a.mult;
-            float nx[BN_HC_MAX_STREAMS];
+    for (int s = 0; s < BN_HC_MAX_STREAMS; ++s) x[s] = s < n ? a.lanes_in[(size_t)s * a.in_stride + at] : 0.f;
+    if (delta) {
+        float y = 0.f;
+        for (int p = 0; p < a.n_slabs; ++p) y += to_f32(delta[(size_t)p * a.slab_stride + at]);
+        y *= a.mult;
+        float nx[BN_HC_MAX_STREAMS];
 #pragma unroll
-            for (int to = 0; to < BN_HC_MAX_STREAMS; ++to) {
-                if (to >= n) { nx[to] = 0.f; continue; }
-                float v = 0.f;
+        for (int to = 0; to < BN_HC_MAX_STREAMS; ++to) {
+            float v = 0.f;
 #pragma unroll
-                for (int s = 0; s < BN_HC_MAX_STREAMS; ++s)
-                    if (s < n) v = fmaf(a.mix[s * n + to], x[s], v);
-                nx[to] = fmaf(a.outc[to], y, v);
-            }
+            for (int s = 0; s < BN_HC_MAX_STREAMS; ++s)
+                if (s < n && to < n) v = fmaf(cm[s * n + to], x[s], v);
+            nx[to] = to < n ? fmaf(co[to], y, v) : 0.f;
+        }
 #pragma unroll
-            for (int s = 0; s < BN_HC_MAX_STREAMS; ++s) x[s] = nx[s];
-            if (a.lanes_out) {
-#pragma unroll
-                for (int s = 0; s < BN_HC_MAX_STREAMS; ++s)
-                    if (s < n) a.lanes_out[(size_t)s * a.out_stride + at] = x[s];
-            }
-        } else if (a.lanes_out && a.lanes_out != a.lanes_in) {
+        for (int s = 0; s < BN_HC_MAX_STREAMS; ++s) x[s] = nx[s];
+        if (a.lanes_out) {
 #pragma unroll
             for (int s = 0; s < BN_HC_MAX_STREAMS; ++s)
                 if (s < n) a.lanes_out[(size_t)s * a.out_stride + at] = x[s];
         }
-        if (!h) continue;
-        float u = 0.f;
+    } else if (a.lanes_out && a.lanes_out != a.lanes_in) {
 #pragma unroll
         for (int s = 0; s < BN_HC_MAX_STREAMS; ++s)
-            if (s < n) u = a.inc ? fmaf(a.inc[s], x[s], u) : u + x[s];
-        const float v = a.w ? fmaf(tanhf(alpha * u), a.w[d], a.b[d]) : u;
-        h[(size_t)r * a.D + d] = from_f32<TH>(v);
+            if (s < n) a.lanes_out[(size_t)s * a.out_stride + at] = x[s];
     }
+    if (!h) return;
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < BN_HC_MAX_STREAMS; ++s)
+        if (s < n) u = a.inc ? fmaf(ci[s], x[s], u) : u + x[s];
+    const float v = a.w ? fmaf(tanhf(a.alpha[0] * u), a.w[d], a.b[d]) : u;
+    h[(size_t)r * a.D + d] = from_f32<TH>(v);
 }
 
 // delta_dtype / h_dtype: BN_DT_F32 or BN_DT_BF16.
@@ -102,7 +106,9 @@ extern "C" int bn_hc_step(int delta_dtype, int h_dtype, const float* lanes_in, l
     a.lanes_in = lanes_in; a.lanes_out = lanes_out; a.delta = delta; a.mix = mix; a.outc = outc; a.inc = inc; a.w = w; a.b = b;
     a.alpha = alpha; a.h = h; a.rows = rows; a.in_stride = in_stride; a.out_stride = out_stride; a.slab_stride = slab_stride;
     a.n_rows = n_rows; a.T = T; a.D = D; a.n = n; a.n_slabs = delta ? n_slabs : 0; a.mult = mult;
-    const dim3 grid(n_rows), block(D >= 1024 ? 256 : 128);
+    const int threads = D >= 256 ? 256 : 64;
+    if ((D + threads - 1) / threads > 65535) return BN_ERR_ARG;
+    const dim3 grid(n_rows, (D + threads - 1) / threads), block(threads);
     const bool df = delta_dtype == BN_DT_F32, hf = h_dtype == BN_DT_F32;
     if ((delta_dtype != BN_DT_F32 && delta_dtype != BN_DT_BF16) || (h_dtype != BN_DT_F32 && h_dtype != BN_DT_BF16)) return BN_ERR_DTYPE;
     if (df && hf) hipLaunchKernelGGL((hc_step_kernel<float, float>), grid, block, 0, s, a);

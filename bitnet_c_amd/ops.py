@@ -2186,7 +2186,7 @@ def lru_gates(u: torch.Tensor, wa_t: torch.Tensor, ba: torch.Tensor, wi_t: torch
     blocks = wa_t.shape[0]
     bw = W // max(blocks, 1)
     if (blocks < 1 or W % blocks or tuple(wa_t.shape) != (blocks, bw, bw) or tuple(wi_t.shape) != (blocks, bw, bw)
-            or not (u.is_contiguous() and wa_t.is_contiguous() and wi_t.is_contiguous()) or bw * 32 > 64 * 1024):
+            or not (u.is_contiguous() and wa_t.is_contiguous() and wi_t.is_contiguous()) or bw * 32 + 32768 > 64 * 1024):
         raise KernelError(f"lru_gates: u {tuple(u.shape)} and gate matrices {tuple(wa_t.shape)} / {tuple(wi_t.shape)} do not fit")
     for t, nm in ((ba, "ba"), (bi, "bi"), (c_neg, "c_neg")):
         _dev(t, nm, torch.float32, 1)
