@@ -243,12 +243,12 @@ def _mutirax_configs(z):
     moe = dict(kind="moe", expert=dict(ff=gated // z["top"] // 64 * 64), router=dict(experts=z["experts"], top=z["top"]))
     H = z["heads"]
     par = dict(left=dict(heads=H, kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], conv=4, scale=z["dim"] ** -0.5,
-                         rot=dict(base=500000.0, dims=z["rot_dims"])),
+                         rot=dict(base=1000000.0, dims=z["rot_dims"])),
                right=dict(width=z["right"], blocks=z["right"] // 256, conv=4))
-    gla = dict(heads=H, dim=z["dim"], vdim=z["dim"], tau=16.0, decay_rank=z["rank"])
+    gla = dict(heads=H, dim=z["dim"], vdim=z["dim"], tau=8.0, decay_rank=z["rank"])
     lat = dict(heads=H, dim=z["dim"], rot_dim=z["rot_dims"], vdim=z["dim"], kv_rank=256 - z["rot_dims"], q_rank=z["width"] // 2,
                scale=(z["dim"] + z["rot_dims"]) ** -0.5,
-               rot=dict(base=250000.0, dims=z["rot_dims"], scaling=dict(factor=8.0, original=1024, fast=32.0, slow=1.0)))
+               rot=dict(base=100000.0, dims=z["rot_dims"], scaling=dict(factor=4.0, original=4096, fast=16.0, slow=2.0)))
     stored = z["layers"] - 3
     layers = []
     for i in range(stored):

@@ -82,13 +82,13 @@ class LatentAttention(Part):
 
     def tensors(self):
         D = self.hidden
-        t = {"wuk": ParamSpec((self.H * self.hs, self.rank)),
-             "wuv": ParamSpec((self.o_dim, self.rank)), "wo": ParamSpec((D, self.o_dim))}
         if self.q_rank:
-            t.update({"wdq": ParamSpec((self.q_rank, D)), "dq_norm": ParamSpec((self.q_rank,), "ones"),
-                      "wuq": ParamSpec((self.q_dim, self.q_rank))})
+            t = {"wdq": ParamSpec((self.q_rank, D)), "dq_norm": ParamSpec((self.q_rank,), "ones"),
+                 "wuq": ParamSpec((self.q_dim, self.q_rank))}
         else:
-            t["wq"] = ParamSpec((self.q_dim, D))
+            t = {"wq": ParamSpec((self.q_dim, D))}
+        t.update({"wuk": ParamSpec((self.H * self.hs, self.rank)), "wuv": ParamSpec((self.o_dim, self.rank)),
+                  "wo": ParamSpec((D, self.o_dim))})
         if self.gated:
             t["wg"] = ParamSpec((self.g_dim, D))
         if self.own:

@@ -65,10 +65,10 @@ CONFIGS = {
         _par(6, 1, 8, 1, 0.5, None, 35, 5, 7, _moe(3, 3, 12))], streams=2, loop=(2, 3, 3)),
     # the head sizes of real models: the matrix-core attention kernels and the grouped products take every layer
     "C": _model(211, 128, 1e-6, 0.5, [
-        _lat(4, 32, 32, 32, 96, 48, 0.125, (250000.0, 8.0, 1024, 32.0, 1.0), _moe(8, 2, 64)),
-        _par(4, 2, 64, 4, 0.125, (500000.0, 64), 128, 4, 4, _dense(256, 1.5)),
-        _gla(2, 64, 64, 16.0, _moe(16, 3, 32), rank=16),
-        _par(2, 1, 128, 4, 0.09, (10000.0, 64), 256, 2, 4, _moe(8, 2, 64))], streams=4, loop=(0, 2, 2)),
+        _lat(4, 32, 32, 32, 96, 48, 0.11, (100000.0, 4.0, 2048, 16.0, 2.0), _moe(6, 2, 64)),
+        _par(4, 1, 64, 3, 0.11, (10000.0, 32), 128, 2, 5, _dense(256, 2.0)),
+        _gla(2, 64, 64, 8.0, _moe(16, 3, 32), rank=16),
+        _par(2, 1, 128, 4, 0.09, (10000.0, 64), 256, 2, 4, _moe(6, 2, 64))], streams=4, loop=(0, 2, 2)),
     # ones everywhere and no streams at all: the plain residual, one head, one expert, one block, no loop
     "D": _model(40, 32, 1e-5, 1.0, [
         _gla(1, 8, 8, 1.0, _moe(1, 1, 8), rank=1),

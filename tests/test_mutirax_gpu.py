@@ -196,7 +196,7 @@ def test_the_gates_and_the_chain_of_the_recurrent_unit(W, blocks):
     ba, bi = torch.randn(W, generator=g), torch.randn(W, generator=g)
     lam = 2.0 * torch.randn(W, generator=g)
     lam[0], lam[1] = -12.0, 6.0                                # a next to 1 whatever r is, and a next to 0
-    lens, first = [30, 1, 13], [4, 0, 0]
+    lens, first = [30 if W != 64 else 300, 1, 13], [4, 0, 0]      # one case with many rows
     slots = [3, 1, 0]
     state = torch.zeros(5, W + 2)
     state[1] = 5.0                                            # a former owner's: ignored at position 0
@@ -701,7 +701,7 @@ def test_a_wide_latent_beside_its_rotated_part(tmp_path, dtype):
     """A latent of 192 numbers beside 64 rotated ones: key rows of 256, values of 192, the widths at which the prompt and
     decode steps of the latent mixer run on the matrix cores in bfloat16.  A prompt across a page's border, then decoded."""
     import bitnet_c_amd as bn
-    cfg = _model(59, 64, 1e-5, 0.5, [_lat(3, 16, 64, 24, 192, 40, 0.11, (250000.0, 8.0, 1024, 32.0, 1.0), None)], streams=2)
+    cfg = _model(59, 64, 1e-5, 0.5, [_lat(3, 16, 64, 24, 192, 40, 0.11, (100000.0, 4.0, 2048, 16.0, 2.0), None)], streams=2)
     folder = write_folder(tmp_path / "wide", cfg, 6)
     toks = torch.randint(0, 59, (90,), generator=torch.Generator().manual_seed(4)).tolist()
     want = plain(folder, toks)
@@ -756,7 +756,8 @@ def test_greedy_generation_through_the_entry_point(folders, name, dtype):
         rms = float(logits.pow(2).mean().sqrt())
         for i, tok in enumerate(g[:settled]):
             gap = float(logits[i].max() - logits[i, tok])
-            assert gap <= (1e-4 if dtype == torch.float32 else 8e-2) * rms, (i, gap / rms)
+            # bfloat16: an element of a row may be off by as much as BF16_ELEMENT of the rows' size (see TOL), on either token
+            assert gap <= (1e-4 if dtype == torch.float32 else BF16_ELEMENT) * rms, (i, gap / rms)
     llm.engine.cache.check()
     assert llm.engine.cache.live_slots() == []
 
