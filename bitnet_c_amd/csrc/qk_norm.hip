@@ -19,6 +19,7 @@
 #include <math.h>
 
 #define QKN_WAVES 4
+#define QKN_MAX_WAVES 16         // waves of the one workgroup that takes a whole row (norms over the whole projections)
 #define QKN_PER_LANE (BN_MAX_HEAD_DIM / BN_WAVE)
 
 struct QkNormArgs {
@@ -51,11 +52,11 @@ __device__ __forceinline__ void qkn_sincos(float a, float* sn, float* cs) {
 }
 
 // a workgroup takes QKN_WAVES heads of one row, a wave each; heads 0 .. H-1 are queries, then Hkv keys, then Hkv values.
-// With norms over the whole projections one workgroup takes all heads of a row, its waves in turn: the query heads are
+// With norms over the whole projections one workgroup (of up to QKN_MAX_WAVES waves) takes all heads of a row, its waves in turn: the query heads are
 // rewritten in place, so the sums of squares over the whole projections must have been formed (by all threads, in front
 // of a barrier) before any of them is, and no other workgroup may read the row meanwhile.
 template <typename T>
-__global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNormArgs a) {
+__global__ __launch_bounds__(QKN_MAX_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNormArgs a) {
     __shared__ float scratch[16];
     const int t = blockIdx.x, lane = threadIdx.x & (BN_WAVE - 1), wave = threadIdx.x / BN_WAVE;
     const int pos = a.positions[t];
@@ -75,7 +76,8 @@ __global__ __launch_bounds__(QKN_WAVES * BN_WAVE) void qk_norm_store_kernel(QkNo
     const int rd = a.inv_freq ? a.rope_dims : 0, half = rd / 2;
     const int n_heads = a.H + 2 * a.Hkv;
     const int head0 = a.norm_all ? 0 : blockIdx.y * QKN_WAVES, head1 = a.norm_all ? n_heads : min(n_heads, head0 + QKN_WAVES);
-    for (int head = head0 + wave; head < head1; head += QKN_WAVES) {
+    const int n_waves = blockDim.x / BN_WAVE;
+    for (int head = head0 + wave; head < head1; head += n_waves) {
         const bool is_q = head < a.H, is_k = !is_q && head < a.H + a.Hkv;
         if (is_q || is_k) {
             if (is_k && !a.k_pages) continue;
@@ -159,7 +161,9 @@ extern "C" int bn_qk_norm_store(int dtype, void* qkv, int ld, const int* positio
     a.eps = eps; a.temp_coef = temp_coef; a.temp_every = temp_every; a.v_transposed = v_transposed ? 1 : 0;
     a.norm_all = norm_all ? 1 : 0; a.rope_dims = inv_freq ? rope_dims : 0; a.rope_interleaved = rope_interleaved ? 1 : 0;
     a.v_from_k = v_from_k ? 1 : 0;
-    const dim3 grid(n_tokens, norm_all ? 1 : (H + 2 * Hkv + QKN_WAVES - 1) / QKN_WAVES), block(QKN_WAVES * BN_WAVE);
+    const int n_heads = H + 2 * Hkv;
+    const int waves = norm_all ? (n_heads < QKN_MAX_WAVES ? (n_heads < QKN_WAVES ? QKN_WAVES : n_heads) : QKN_MAX_WAVES) : QKN_WAVES;
+    const dim3 grid(n_tokens, norm_all ? 1 : (n_heads + QKN_WAVES - 1) / QKN_WAVES), block(waves * BN_WAVE);
     if (dtype == BN_DT_F32) hipLaunchKernelGGL(qk_norm_store_kernel<float>, grid, block, 0, s, a);
     else if (dtype == BN_DT_BF16) hipLaunchKernelGGL(qk_norm_store_kernel<bf16>, grid, block, 0, s, a);
     else return BN_ERR_DTYPE;

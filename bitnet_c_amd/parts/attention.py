@@ -178,7 +178,8 @@ class Attention(Part):
             if not kv.writes:
                 raise ValueError("attention: a convolution on the projections needs the layer's own keys")
             seqs = dict(seq_lens=ctx.seq_lens) if ctx.is_decode else dict(tiles=ctx.tiles(ops.SEQUENCE_TILE))
-            qk = ops.short_conv(qkv, 0, self.conv_w, None, kv.state, ctx.positions, ctx.seq_index, ctx.slot_ids, **seqs)
+            state = kv.state if kv.state is not None else self._no_state(qkv.device)     # one tap keeps nothing
+            qk = ops.short_conv(qkv, 0, self.conv_w, None, state, ctx.positions, ctx.seq_index, ctx.slot_ids, **seqs)
             if self.value_is_key:
                 qkv = qk
             else:
@@ -227,6 +228,12 @@ class Attention(Part):
 
     def _sink(self):
         return self.sink_values if self.sink_learned else self.sink
+
+    def _no_state(self, device):
+        """What a convolution of one tap is handed for a state when the entry has none: it is never read."""
+        if getattr(self, "_empty_state", None) is None:
+            self._empty_state = torch.zeros((1, 1), dtype=torch.float32, device=device)
+        return self._empty_state
 
     def forward(self, h, ctx, kv, lazy_ok: bool = False):
         if self.general:
