@@ -300,6 +300,15 @@ struct GlaArgs {
     long long state_stride;
     int ld, q_col, k_col, v_col, H, dk, dv;
     float q_scale, inv_tau;
+    // Long prompts in pieces that run side by side (phase > 0): a sequence's tokens are cut into pieces of `piece`; every
+    // (sequence, piece) has a [H][dk][dv] matrix in `carry` and a [H][dk] row in `fade`.
+    //   phase 1  every piece from nothing: its own sum of decayed k v^T into carry (no outputs)
+    //   (bn_gla_fade: the product of a piece's decays per key channel; bn_gla_carry: S_in of every piece from the
+    //    sequence's state, the pieces' sums and fades in order, left in carry; the sequence's state after its last piece)
+    //   phase 2  every piece from its S_in: the outputs
+    int phase, piece, max_pieces;
+    float* carry;
+    float* fade;
 };
 
 // A wave owns (sequence, head, 16 value columns); a workgroup is NW such waves over neighbouring columns of one head, so
@@ -320,19 +329,29 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
     constexpr int PF = (RUN * DKP + NT - 1) / NT, PV = (RUN * VC + NT - 1) / NT;
     __shared__ __align__(16) float q_s[2][RUN][DKL], k_s[2][RUN][DKL], a_s[2][RUN][DKL];
     __shared__ float v_s[2][RUN][VC];
-    const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x);
+    SeqRange sr = seq_range(a.tiles, a.seq_lens, a.phase ? blockIdx.x / a.max_pieces : blockIdx.x);
     if (sr.n <= 0 || sr.pos0 < 0) return;
     const int head = blockIdx.y, colb = blockIdx.z * VC;
+    float* carry = nullptr;
+    if (a.phase) {                                        // this workgroup's piece of the sequence
+        const int first = (blockIdx.x % a.max_pieces) * a.piece;
+        if (first >= sr.n) return;
+        carry = a.carry + ((size_t)blockIdx.x * a.H + head) * a.dk * a.dv;
+        sr.row0 += first;
+        sr.n = min(a.piece, sr.n - first);
+    }
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, sl = lane >> 4, c = lane & 15;
     const int col = colb + wave * GLA_COLS + c;
     const bool has = col < a.dv;
     const T* x = reinterpret_cast<const T*>(a.x);
-    float* sp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * a.dk * a.dv + (has ? col : 0);
+    float* sp = a.phase ? carry + (has ? col : 0)
+                        : a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * a.dk * a.dv + (has ? col : 0);
     float S[RPL];
 #pragma unroll
     for (int r = 0; r < RPL; ++r) {
         const int i = sl * RPL + r;
-        S[r] = (sr.pos0 > 0 && has && i < a.dk) ? sp[(size_t)i * a.dv] : 0.f;
+        const bool from_memory = a.phase == 2 || (a.phase == 0 && sr.pos0 > 0);
+        S[r] = (from_memory && has && i < a.dk) ? sp[(size_t)i * a.dv] : 0.f;
     }
     float rq[PF], rk[PF], rz[PF], rv[PV];
     // loads from clamped places, unconditional: what lies outside the run or the head is never parked
@@ -413,18 +432,53 @@ __global__ __launch_bounds__(BN_WAVE * NW) void gla_scan_kernel(GlaArgs a) {
             float v = o[tt];
             v += __shfl_xor(v, 16, BN_WAVE);
             v += __shfl_xor(v, 32, BN_WAVE);
-            if (tt < run && sl == 0 && has) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col] = v;
+            if (tt < run && sl == 0 && has && a.phase != 1) a.o[(size_t)(sr.row0 + t0 + tt) * (a.H * a.dv) + (size_t)head * a.dv + col] = v;
         }
         if (more) park(buf ^ 1, t0 + RUN);
         __syncthreads();
     }
-    if (has) {
+    if (has && a.phase != 2) {
 #pragma unroll
         for (int r = 0; r < RPL; ++r) {
             const int i = sl * RPL + r;
             if (i < a.dk) sp[(size_t)i * a.dv] = S[r];
         }
     }
+}
+
+// The product of a piece's decays per key channel, as the exponential of the sum of their logarithms.
+__global__ __launch_bounds__(256) void gla_fade_kernel(GlaArgs a) {
+    const SeqRange sr = seq_range(a.tiles, a.seq_lens, blockIdx.x / a.max_pieces);
+    const int first = (blockIdx.x % a.max_pieces) * a.piece, ch = blockIdx.y * blockDim.x + threadIdx.x;
+    if (sr.n <= 0 || sr.pos0 < 0 || first >= sr.n || ch >= a.H * a.dk) return;
+    const int n = min(a.piece, sr.n - first);
+    const float* z = a.z + (size_t)(sr.row0 + first) * (a.H * a.dk) + ch;
+    float sum = 0.f;
+    for (int t = 0; t < n; ++t) {
+        const float zz = z[(size_t)t * (a.H * a.dk)];
+        sum += (fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)))) * a.inv_tau;
+    }
+    a.fade[(size_t)blockIdx.x * (a.H * a.dk) + ch] = expf(sum);
+}
+
+// One thread an element of a head's matrix: it walks the sequence's pieces in order, leaves in carry what every piece
+// starts from, and in the state what the sequence ends with.
+__global__ __launch_bounds__(256) void gla_carry_kernel(GlaArgs a) {
+    const int tile = blockIdx.x, head = blockIdx.y, e = blockIdx.z * blockDim.x + threadIdx.x;
+    const SeqRange sr = seq_range(a.tiles, a.seq_lens, tile);
+    if (sr.n <= 0 || sr.pos0 < 0 || e >= a.dk * a.dv) return;
+    const int i = e / a.dv;
+    float* sp = a.state + (size_t)a.slot_ids[sr.seq] * a.state_stride + (size_t)head * a.dk * a.dv + e;
+    float S = sr.pos0 > 0 ? *sp : 0.f;
+    const int pieces = (sr.n + a.piece - 1) / a.piece;
+    for (int p = 0; p < pieces; ++p) {
+        const size_t at = (size_t)tile * a.max_pieces + p;
+        float* c = a.carry + (at * a.H + head) * a.dk * a.dv + e;
+        const float own = *c, f = a.fade[(at * a.H + head) * a.dk + i];
+        *c = S;
+        S = fmaf(f, S, own);
+    }
+    *sp = S;
 }
 
 extern "C" int bn_gla_supports(int dk, int dv) { return (dk >= 1 && dk <= GLA_MAX_DIM && dv >= 1) ? 1 : 0; }
@@ -435,7 +489,7 @@ static int gla_waves(int dv) { return dv <= GLA_COLS ? 1 : 4; }
 
 template <typename T, int NW>
 static int gla_launch_nw(const GlaArgs& a, int n_seqs, hipStream_t s) {
-    const dim3 grid(n_seqs, a.H, (a.dv + GLA_COLS * NW - 1) / (GLA_COLS * NW)), block(BN_WAVE * NW);
+    const dim3 grid(a.phase ? n_seqs * a.max_pieces : n_seqs, a.H, (a.dv + GLA_COLS * NW - 1) / (GLA_COLS * NW)), block(BN_WAVE * NW);
     const int rpl = (a.dk + GLA_SLICES - 1) / GLA_SLICES;
     if (rpl <= 8) hipLaunchKernelGGL((gla_scan_kernel<T, 8, NW>), grid, block, 0, s, a);
     else if (rpl <= 16) hipLaunchKernelGGL((gla_scan_kernel<T, 16, NW>), grid, block, 0, s, a);
@@ -462,7 +516,34 @@ extern "C" int bn_gla_scan(int dtype, const void* x, int ld, int q_col, int k_co
     a.x = x; a.z = z; a.o = o; a.state = state; a.tiles = tiles; a.seq_lens = seq_lens; a.slot_ids = slot_ids;
     a.state_stride = state_stride; a.ld = ld; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col; a.H = H; a.dk = dk; a.dv = dv;
     a.q_scale = q_scale; a.inv_tau = inv_tau;
+    a.phase = 0; a.piece = 0; a.max_pieces = 1; a.carry = nullptr; a.fade = nullptr;
     if (dtype == BN_DT_F32) return gla_launch<float>(a, n_seqs, s);
     if (dtype == BN_DT_BF16) return gla_launch<bf16>(a, n_seqs, s);
     return BN_ERR_DTYPE;
+}
+
+// The same over long prompts, their pieces side by side (prompt form only).  carry: [n_tiles max_pieces, H dk dv] and
+// fade: [n_tiles max_pieces, H dk] float32 work space; max_pieces covers the longest sequence's pieces.  A sequence's
+// outputs and state differ from the plain walk's by rounding alone (a piece's own sum is formed from nothing and joined
+// to what came before it by one multiplication and addition).
+extern "C" int bn_gla_scan_pieces(int dtype, const void* x, int ld, int q_col, int k_col, int v_col, const float* z, float* o,
+                                  float* state, long long state_stride, const int* tiles, int n_tiles, const int* slot_ids, int H,
+                                  int dk, int dv, float q_scale, float inv_tau, int piece, int max_pieces, float* carry,
+                                  float* fade, hipStream_t s) {
+    if (n_tiles <= 0 || H <= 0 || !bn_gla_supports(dk, dv) || !x || !z || !o || !state || !slot_ids || !tiles || !carry || !fade) return BN_ERR_ARG;
+    if (ld < q_col + H * dk || ld < k_col + H * dk || ld < v_col + H * dv || state_stride < (long long)H * dk * dv) return BN_ERR_ARG;
+    if (piece < 1 || max_pieces < 1 || H > 65535 || (long long)n_tiles * max_pieces > 0x7fffffffLL) return BN_ERR_ARG;
+    if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
+    GlaArgs a;
+    a.x = x; a.z = z; a.o = o; a.state = state; a.tiles = tiles; a.seq_lens = nullptr; a.slot_ids = slot_ids;
+    a.state_stride = state_stride; a.ld = ld; a.q_col = q_col; a.k_col = k_col; a.v_col = v_col; a.H = H; a.dk = dk; a.dv = dv;
+    a.q_scale = q_scale; a.inv_tau = inv_tau; a.piece = piece; a.max_pieces = max_pieces; a.carry = carry; a.fade = fade;
+    a.phase = 1;
+    int rc = dtype == BN_DT_F32 ? gla_launch<float>(a, n_tiles, s) : gla_launch<bf16>(a, n_tiles, s);
+    if (rc != 0) return rc;
+    hipLaunchKernelGGL(gla_fade_kernel, dim3(n_tiles * max_pieces, (H * dk + 255) / 256), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(gla_carry_kernel, dim3(n_tiles, H, (dk * dv + 255) / 256), dim3(256), 0, s, a);
+    if ((rc = bn_launch_status()) != 0) return rc;
+    a.phase = 2;
+    return dtype == BN_DT_F32 ? gla_launch<float>(a, n_tiles, s) : gla_launch<bf16>(a, n_tiles, s);
 }

@@ -98,6 +98,8 @@ _SIGNATURES = {
         "bn_gla_supports": [c_int, c_int],
         "bn_gla_scan": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int,
                         c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p],
+        "bn_gla_scan_pieces": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p,
+                               c_int, c_void_p, c_int, c_int, c_int, c_float, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p],
     },
     "lightning": {
         "bn_lightning_supports": [c_int, c_int],
@@ -2227,12 +2229,20 @@ def gla_supported(dk: int, dv: int) -> bool:
     return bool(_fn("conv_scans", "bn_gla_supports")(int(dk), int(dv)))
 
 
+GLA_PIECE = 64                  # tokens of a piece of a long prompt
+GLA_PIECES_MIN_ROWS = 256       # prompt steps of at least this many rows walk their sequences in pieces side by side
+
+
 def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tensor, state: torch.Tensor, slot_ids, H: int,
-             dk: int, dv: int, q_scale: float, inv_tau: float, *, tiles=None, seq_lens=None) -> torch.Tensor:
+             dk: int, dv: int, q_scale: float, inv_tau: float, *, tiles=None, seq_lens=None, pieces: Optional[bool] = None) -> torch.Tensor:
     """Gated linear attention over every sequence's tokens: per head S <- diag(alpha_t) S + k_t v_t^T, o_t = S^T (q_scale q_t)
     with alpha = sigmoid(z)^inv_tau per key channel.  x [T, ld] holds q at q_col, k at k_col (heads of dk) and v at v_col
     (heads of dv); z [T, H dk] float32.  state: float32 [slots, >= H dk dv], a head's matrix [dk, dv] row-major; zeros at
-    position 0.  Returns o [T, H dv] float32."""
+    position 0.  Returns o [T, H dv] float32.
+    pieces (prompt form): cut every sequence into pieces of GLA_PIECE tokens that are walked side by side: every piece's
+    own sum from nothing, the sequence's state carried through the pieces' sums and the products of their decays, then
+    every piece's outputs from what it starts with.  Twice the arithmetic on many times the workgroups; the results differ
+    from the plain walk's by rounding alone.  None: for steps of at least GLA_PIECES_MIN_ROWS rows."""
     require_gpu()
     _dev(x, "x", dims=2)
     _dev(z, "z", torch.float32, 2)
@@ -2244,6 +2254,18 @@ def gla_scan(x: torch.Tensor, q_col: int, k_col: int, v_col: int, z: torch.Tenso
     _dev(slot_ids, "slot_ids", torch.int32, 1)
     tl, n_seqs, sl = _seq_args(tiles, seq_lens, "gla_scan")
     o = torch.empty((T, H * dv), dtype=torch.float32, device=x.device)
+    if pieces is None:                                   # long steps, as long as the pieces' matrices stay below 2 GB
+        pieces = (tl is not None and T >= GLA_PIECES_MIN_ROWS
+                  and n_seqs * -(-T // GLA_PIECE) * H * dk * dv * 4 <= 2 << 30)
+    if pieces and tl is not None and T and n_seqs:
+        max_pieces = -(-T // GLA_PIECE)                  # no sequence of the step has more rows than the step
+        carry = torch.empty((n_seqs * max_pieces, H * dk * dv), dtype=torch.float32, device=x.device)
+        fade = torch.empty((n_seqs * max_pieces, H * dk), dtype=torch.float32, device=x.device)
+        _check(_fn("conv_scans", "bn_gla_scan_pieces")(_code(x.dtype), x.data_ptr(), _rows(x, "x"), int(q_col), int(k_col), int(v_col),
+                                                       z.data_ptr(), o.data_ptr(), state.data_ptr(), stride, tl, n_seqs,
+                                                       slot_ids.data_ptr(), H, dk, dv, float(q_scale), float(inv_tau), GLA_PIECE,
+                                                       max_pieces, carry.data_ptr(), fade.data_ptr(), _stream()), "gla_scan(pieces)")
+        return o
     if T and n_seqs:
         _check(_fn("conv_scans", "bn_gla_scan")(_code(x.dtype), x.data_ptr(), _rows(x, "x"), int(q_col), int(k_col), int(v_col),
                                                 z.data_ptr(), o.data_ptr(), state.data_ptr(), stride, tl, n_seqs, sl,

@@ -292,11 +292,14 @@ def test_gated_linear_attention_over_prompts_portions_and_single_tokens(dtype, H
         r += n
     tiles.append([0, 0, 0, 0])
     x, z = torch.cat([t[:-1] for t in xs]).to(DEV), f32(torch.cat([t[:-1] for t in zs]))
-    o = ops.gla_scan(x, qc, kc, vc, z, st, i32(slots), H, dk, dv, dk ** -0.5, 1.0 / tau, tiles=i32(tiles))
     tol = 2e-5
-    assert rel_err(o, torch.cat([w[:-1] for w in want]).reshape(sum(lens), -1)) < tol
-    for bq in range(3):
-        assert rel_err(st[slots[bq], :H * dk * dv], S_after[bq].reshape(-1)) < tol
+    for pieces in (True, False):                       # long prompts' form (pieces of 64 tokens side by side), then the plain walk
+        st = state.to(DEV)
+        o = ops.gla_scan(x, qc, kc, vc, z, st, i32(slots), H, dk, dv, dk ** -0.5, 1.0 / tau, tiles=i32(tiles), pieces=pieces)
+        assert rel_err(o, torch.cat([w[:-1] for w in want]).reshape(sum(lens), -1)) < tol, pieces
+        for bq in range(3):
+            assert rel_err(st[slots[bq], :H * dk * dv], S_after[bq].reshape(-1)) < tol, pieces
+        assert torch.equal(st[[0, 3, 5]].cpu(), state[[0, 3, 5]]) and torch.equal(st[:, H * dk * dv:].cpu(), state[:, H * dk * dv:])
     xd = torch.stack([xs[2][-1], xs[0][-1], torch.zeros(Wd, dtype=dtype), xs[1][-1]]).to(DEV)
     zd = f32(torch.stack([zs[2][-1], zs[0][-1], torch.zeros(H * dk), zs[1][-1]]))
     before = st.clone()
