@@ -272,6 +272,82 @@ __global__ __launch_bounds__(64) void lru_scan_kernel(const float* __restrict__ 
     *sp = S;
 }
 
+// Long prompts in pieces side by side, as the gated linear attention's: a thread owns (sequence, piece, channel).
+//   phase 1  the piece's own chain from nothing and the product of its decays -> carry[.][0 / 1][channel]
+//   carry    the sequence's S through the pieces in order; carry[.][0] then holds what a piece starts from
+//   phase 2  the piece's chain from there, the outputs
+template <typename T>
+__global__ __launch_bounds__(64) void lru_scan_pieces_kernel(const float* __restrict__ av, const float* __restrict__ bv,
+                                                             const T* __restrict__ ypre, int ldy, T* __restrict__ out,
+                                                             float* __restrict__ carry, const int* __restrict__ tiles, int W,
+                                                             int piece, int max_pieces, int phase) {
+    SeqRange sr = seq_range(tiles, nullptr, blockIdx.x / max_pieces);
+    const int c = blockIdx.y * blockDim.x + threadIdx.x, first = (blockIdx.x % max_pieces) * piece;
+    if (sr.n <= 0 || sr.pos0 < 0 || first >= sr.n || c >= W) return;
+    const int n = min(piece, sr.n - first), row0 = sr.row0 + first;
+    float* cp = carry + (size_t)blockIdx.x * 2 * W + c;
+    float S = phase == 2 ? cp[0] : 0.f, P = 1.0f;
+    const float* ap = av + (size_t)row0 * W + c;
+    const float* bp = bv + (size_t)row0 * W + c;
+    const T* yp = ypre + (size_t)row0 * ldy + c;
+    T* op = out + (size_t)row0 * W + c;
+    for (int t0 = 0; t0 < n; t0 += LRU_AHEAD) {
+        float a[LRU_AHEAD], b[LRU_AHEAD], y[LRU_AHEAD];
+#pragma unroll
+        for (int i = 0; i < LRU_AHEAD; ++i) {
+            const int t = min(t0 + i, n - 1);
+            a[i] = ap[(size_t)t * W]; b[i] = bp[(size_t)t * W]; y[i] = phase == 2 ? to_f32(yp[(size_t)t * ldy]) : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < LRU_AHEAD; ++i) {
+            if (t0 + i >= n) break;
+            S = fmaf(a[i], S, b[i]);
+            if (phase == 2) op[(size_t)(t0 + i) * W] = from_f32<T>(S * bn_gate_act(y[i], BN_ACT_GELU_TANH));
+            else P *= a[i];
+        }
+    }
+    if (phase == 1) { cp[0] = S; cp[W] = P; }
+}
+
+__global__ __launch_bounds__(64) void lru_carry_kernel(float* __restrict__ carry, float* __restrict__ state, long long state_stride,
+                                                       const int* __restrict__ tiles, const int* __restrict__ slot_ids, int W,
+                                                       int piece, int max_pieces) {
+    const SeqRange sr = seq_range(tiles, nullptr, blockIdx.x);
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (sr.n <= 0 || sr.pos0 < 0 || c >= W) return;
+    float* sp = state + (size_t)slot_ids[sr.seq] * state_stride + c;
+    float S = sr.pos0 > 0 ? *sp : 0.f;
+    const int pieces = (sr.n + piece - 1) / piece;
+    for (int p = 0; p < pieces; ++p) {
+        float* cp = carry + ((size_t)blockIdx.x * max_pieces + p) * 2 * W + c;
+        const float own = cp[0], f = cp[W];
+        cp[0] = S;
+        S = fmaf(f, S, own);
+    }
+    *sp = S;
+}
+
+// carry: [n_tiles max_pieces, 2, W] float32 work space.  Results differ from bn_lru_scan's by rounding alone.
+extern "C" int bn_lru_scan_pieces(int dtype, const float* av, const float* bv, const void* ypre, int ldy, void* out, float* state,
+                                  long long state_stride, const int* tiles, int n_tiles, const int* slot_ids, int W, int piece,
+                                  int max_pieces, float* carry, hipStream_t s) {
+    if (n_tiles <= 0 || W <= 0 || !av || !bv || !ypre || !out || !state || !slot_ids || !tiles || !carry || ldy < W) return BN_ERR_ARG;
+    if (state_stride < W || piece < 1 || max_pieces < 1 || (long long)n_tiles * max_pieces > 0x7fffffffLL) return BN_ERR_ARG;
+    if (dtype != BN_DT_F32 && dtype != BN_DT_BF16) return BN_ERR_DTYPE;
+    const dim3 grid(n_tiles * max_pieces, (W + 63) / 64), cgrid(n_tiles, (W + 63) / 64);
+    for (int phase = 1; phase <= 2; ++phase) {
+        if (dtype == BN_DT_F32)
+            hipLaunchKernelGGL(lru_scan_pieces_kernel<float>, grid, dim3(64), 0, s, av, bv, (const float*)ypre, ldy, (float*)out, carry,
+                               tiles, W, piece, max_pieces, phase);
+        else
+            hipLaunchKernelGGL(lru_scan_pieces_kernel<bf16>, grid, dim3(64), 0, s, av, bv, (const bf16*)ypre, ldy, (bf16*)out, carry,
+                               tiles, W, piece, max_pieces, phase);
+        if (phase == 1)
+            hipLaunchKernelGGL(lru_carry_kernel, cgrid, dim3(64), 0, s, carry, state, state_stride, tiles, slot_ids, W, piece, max_pieces);
+    }
+    return bn_launch_status();
+}
+
 extern "C" int bn_lru_scan(int dtype, const float* av, const float* bv, const void* ypre, int ldy, void* out, float* state,
                            long long state_stride, const int* tiles, int n_seqs, const int* seq_lens, const int* slot_ids,
                            int W, hipStream_t s) {

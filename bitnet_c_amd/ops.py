@@ -95,6 +95,8 @@ _SIGNATURES = {
                          c_void_p],
         "bn_lru_scan": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p,
                         c_void_p, c_int, c_void_p],
+        "bn_lru_scan_pieces": [c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_longlong, c_void_p, c_int, c_void_p,
+                               c_int, c_int, c_int, c_void_p, c_void_p],
         "bn_gla_supports": [c_int, c_int],
         "bn_gla_scan": [c_int, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p, c_int,
                         c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p],
@@ -2203,10 +2205,11 @@ def lru_gates(u: torch.Tensor, wa_t: torch.Tensor, ba: torch.Tensor, wi_t: torch
 
 
 def lru_scan(a: torch.Tensor, b: torch.Tensor, y_pre: torch.Tensor, state: torch.Tensor, slot_ids, *, tiles=None,
-             seq_lens=None) -> torch.Tensor:
+             seq_lens=None, pieces: Optional[bool] = None) -> torch.Tensor:
     """S <- a_t S + b_t per channel over every sequence's tokens (a, b [T, W] float32; S from the sequence's state row,
     zeros at position 0, left there afterwards), the result times gelu_tanh(y_pre) (y_pre [T, W] in the activations'
-    type, which is the result's)."""
+    type, which is the result's).  pieces (prompt form): as gla_scan's, with pieces of LRU_PIECE tokens; None: for steps of
+    at least GLA_PIECES_MIN_ROWS rows."""
     require_gpu()
     _dev(a, "a", torch.float32, 2)
     _dev(b, "b", torch.float32, 2)
@@ -2218,6 +2221,16 @@ def lru_scan(a: torch.Tensor, b: torch.Tensor, y_pre: torch.Tensor, state: torch
     _dev(slot_ids, "slot_ids", torch.int32, 1)
     tl, n_seqs, sl = _seq_args(tiles, seq_lens, "lru_scan")
     out = torch.empty((T, W), dtype=y_pre.dtype, device=a.device)
+    if pieces is None:
+        pieces = tl is not None and T >= GLA_PIECES_MIN_ROWS
+    if pieces and tl is not None and T and n_seqs:
+        max_pieces = -(-T // LRU_PIECE)
+        carry = torch.empty((n_seqs * max_pieces, 2, W), dtype=torch.float32, device=a.device)
+        _check(_fn("conv_scans", "bn_lru_scan_pieces")(_code(y_pre.dtype), a.data_ptr(), b.data_ptr(), y_pre.data_ptr(),
+                                                       _rows(y_pre, "y_pre"), out.data_ptr(), state.data_ptr(), stride, tl, n_seqs,
+                                                       slot_ids.data_ptr(), W, LRU_PIECE, max_pieces, carry.data_ptr(), _stream()),
+               "lru_scan(pieces)")
+        return out
     if T and n_seqs:
         _check(_fn("conv_scans", "bn_lru_scan")(_code(y_pre.dtype), a.data_ptr(), b.data_ptr(), y_pre.data_ptr(), _rows(y_pre, "y_pre"),
                                                 out.data_ptr(), state.data_ptr(), stride, tl, n_seqs, sl, slot_ids.data_ptr(), W,
@@ -2230,6 +2243,7 @@ def gla_supported(dk: int, dv: int) -> bool:
 
 
 GLA_PIECE = 64                  # tokens of a piece of a long prompt
+LRU_PIECE = 64                  # the same for the recurrent unit's chain
 GLA_PIECES_MIN_ROWS = 256       # prompt steps of at least this many rows walk their sequences in pieces side by side
 
 

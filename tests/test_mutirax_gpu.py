@@ -234,10 +234,11 @@ def test_the_gates_and_the_chain_of_the_recurrent_unit(W, blocks):
     for bq, n in enumerate(lens):
         tiles.append([bq, r, n, first[bq]])
         r += n
-    st = state.to(DEV)
     wide = torch.cat([torch.cat([x[:-1] for x in ys]), torch.zeros(r, 3)], dim=1).to(DEV)     # y: columns of a wider tensor
-    out = ops.lru_scan(a_dev, b_dev, wide[:, :W], st, i32(slots), tiles=i32(tiles))
-    assert rel_err(out, torch.cat([x[:-1] for x in want])) < 2e-5
+    for pieces in (True, False):                       # long prompts' form (pieces side by side), then the plain walk
+        st = state.to(DEV)
+        out = ops.lru_scan(a_dev, b_dev, wide[:, :W], st, i32(slots), tiles=i32(tiles), pieces=pieces)
+        assert rel_err(out, torch.cat([x[:-1] for x in want])) < 2e-5, pieces
     ud = torch.stack([us[2][-1], us[0][-1], us[1][-1]])
     a_dev, b_dev = ops.lru_gates(f32(ud), wa_t, f32(ba), wi_t, f32(bi), f32(c_neg))
     yd = torch.stack([ys[2][-1], ys[0][-1], ys[1][-1]]).to(DEV)
