@@ -256,7 +256,7 @@ def test_gated_linear_attention_over_prompts_portions_and_single_tokens(dtype, H
     from bitnet_c_amd import ops
     g = torch.Generator().manual_seed(dk * 7 + dv)
     tau = 3.0
-    lens, first = [37, 1, 70], [5, 0, 0]
+    lens, first = ([37, 1, 70], [5, 0, 0]) if dk != 32 else ([201, 64, 130], [9, 0, 0])    # pieces: two; four, one whole, three
     qc, kc, vc, Wd = 3, 3 + H * dk + 2, 3 + 2 * H * dk + 4, 3 + 2 * H * dk + 4 + H * dv + 1
     slots = [4, 1, 2]
     state = torch.zeros(6, H * dk * dv + 3)
